@@ -41,7 +41,9 @@ enum ndist_status {
     NDIST_ERR_BAD_SHAPE = 2,      /* non-positive size, CI or CO not divisible by G, or a size product overflowing int32 */
     NDIST_ERR_BAD_P = 3,          /* p <= 0, NaN, or infinite where a finite p is required */
     NDIST_ERR_HIP = 4,            /* a HIP runtime call failed; see ndist_last_hip_error() */
-    NDIST_ERR_NO_DEVICE = 5       /* no HIP device is usable */
+    NDIST_ERR_NO_DEVICE = 5,      /* no HIP device is usable */
+    NDIST_ERR_CAPTURE = 6         /* the stream is being captured into a HIP graph and the call needs temporary device
+                                     memory from the library's arenas: nothing was allocated or launched */
 };
 
 /* Library version (major * 10000 + minor * 100 + patch). */
@@ -72,6 +74,12 @@ void ndist_set_skip_mode(int skip, int bounds);
  * allocate nor wait for the stream once warmed up.  This call frees the arenas that no running call is using; it
  * waits for the device.  Returns a status code. */
 int ndist_release_scratch(void);
+/* Test aid, no counterpart in the reference: hipMalloc / hipFree calls the library has made for its arenas since it
+ * was loaded (either pointer may be NULL).  Unchanged across a call = that call allocated nothing. */
+void ndist_scratch_counters(long* mallocs, long* frees);
+/* HIP graphs: an entry point that would take arena scratch returns NDIST_ERR_CAPTURE when `stream` is being captured
+ * (before it allocates or launches anything): a captured graph must not hold addresses of memory a later call may
+ * free.  Entry points and shapes that need no scratch can be captured. */
 
 /* ---- finite p: replaces template struct norm_dist<ip> (core/cuda/norm_dist.h:4-14) ------------------- */
 

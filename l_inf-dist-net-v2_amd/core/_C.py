@@ -45,6 +45,8 @@ _lib.ndist_release_scratch.argtypes = []
 _lib.ndist_release_scratch.restype = ctypes.c_int
 _lib.ndist_last_kernel_ms.argtypes = [ctypes.POINTER(ctypes.c_float)]
 _lib.ndist_last_kernel_ms.restype = ctypes.c_int
+_lib.ndist_scratch_counters.argtypes = [ctypes.POINTER(ctypes.c_long), ctypes.POINTER(ctypes.c_long)]
+_lib.ndist_scratch_counters.restype = None
 
 _DIMS = (_I, _I, _I, _I, _I)
 _norm_fwd = _sig("ndist_norm_dist_forward", _P, _P, *_DIMS, _P, _F, _P)
@@ -71,8 +73,27 @@ _conv_bnd_bwd_x = _sig("ndist_conv_bound_inf_dist_backward_input", _P, _P, _P, _
 _conv_bnd_bwd_xw = _sig("ndist_conv_bound_inf_dist_backward_input_weight", _P, _P, _P, _P, *([_I] * 14), _P, _P, _P, _P)
 
 
+# status codes of the library (include/norm_dist_hip.h)
+ERR_CAPTURE = 6
+
+
+class NormDistError(RuntimeError):
+    """A library call returned a non-zero status; `status` holds the code."""
+
+    def __init__(self, message, status):
+        super().__init__(message)
+        self.status = status
+
+
 def version():
     return _lib.ndist_version()
+
+
+def scratch_counters():
+    """(hipMalloc calls, hipFree calls) the library has made for its scratch arenas since it was loaded."""
+    m, f = ctypes.c_long(0), ctypes.c_long(0)
+    _lib.ndist_scratch_counters(ctypes.byref(m), ctypes.byref(f))
+    return m.value, f.value
 
 
 def set_profiling(enable):
@@ -119,13 +140,14 @@ def _check(dtype, **tensors):
     return dev
 
 
-def _run(fn, dev, *args):
+def _run(fn, dev, *args, stream=None):
     with torch.cuda.device(dev):
-        stream = torch.cuda.current_stream(dev).cuda_stream
+        if stream is None:
+            stream = torch.cuda.current_stream(dev).cuda_stream
         rc = fn(*args, stream)
     if rc != 0:
-        raise RuntimeError("%s failed: %s (hip error %d)" % (
-            fn.__name__, _lib.ndist_status_string(rc).decode(), _lib.ndist_last_hip_error()))
+        raise NormDistError("%s failed: %s (hip error %d)" % (
+            fn.__name__, _lib.ndist_status_string(rc).decode(), _lib.ndist_last_hip_error()), rc)
 
 
 def _p(t):

@@ -206,17 +206,24 @@ __global__ __launch_bounds__(kBoundProbeBlock) void bwd_bound_probe_kernel(const
 // geometry (M rows, HW = 1); the factors are indexed by row in both geometries.
 constexpr int kBwdTransposeMinHW = 16;
 
-int launch_norm_backward(const float* gout, const float* x, const float* w, const float* out, const Geom& s, float* gx,
-                         float* gw, float p, hipStream_t st) {
+// What the launcher decides from the shape and the exponent alone.
+struct BwdPlan {
+    int ip;              // exponent variant of the kernels
+    int cfg;             // 0..2: row-split workgroups of 16 / 8 / 4 waves; 3: small-batch kernel
+    int rows_per_wg;
+    bool want_adaptive;  // large exponent on a problem worth the probes: skipping and plain variants are all queued
+};
+static BwdPlan plan_backward(const Geom& s, float p) {
     const float q = p - 1.0f;
-    int ip = q >= 1.0f ? -1 : -2;  // general exponent; below 1 grad_output is not folded into the factor
-    if (q == (float)(int)q && (int)q >= 0 && (int)q <= 8) ip = (int)q;  // as far as the reference's ladder goes
+    BwdPlan pl{};
+    pl.ip = q >= 1.0f ? -1 : -2;  // general exponent; below 1 grad_output is not folded into the factor
+    if (q == (float)(int)q && (int)q >= 0 && (int)q <= 8) pl.ip = (int)q;  // as far as the reference's ladder goes
     // 3: small-batch kernel (waves split co, 32-row chunks); its grid index must fit 32 bits
     const bool small = s.M <= kBwdSmallMaxM && (long)s.G * ceil_div(s.CIg, kBwdSlab) * ceil_div(s.M, kBwdSmallRows) * 64 < (1L << 31);
     // Large exponents on problems worth the extra launches: the skipping variants (IP -3, -4) and the plain one
     // (IP -1) are all queued and device-side probes of the data open the gate of one of them.
-    const bool want_adaptive = ip == -1 && q >= 15.0f && ((double)s.M * s.COg * s.G * s.CIg >= 2e8 || skip_forced_on());
-    int cfg = 3;
+    pl.want_adaptive = pl.ip == -1 && q >= 15.0f && ((double)s.M * s.COg * s.G * s.CIg >= 2e8 || skip_forced_on());
+    pl.cfg = 3;
     if (!small) {
         // rows are padded to whole chunks of a workgroup's rows (512, 256 or 128): the configuration with the least
         // padded work wins; measured cost of one chunk relative to the 512-row one: 1, 0.505, 0.28.  The bounds
@@ -226,11 +233,27 @@ int launch_norm_backward(const float* gout, const float* x, const float* w, cons
         constexpr double kChunkCost[2][3] = {{1.0, 0.505, 0.28}, {1.0, 0.63, 0.44}};
         double best = 0.0;
         for (int c = 0; c < 3; c++) {
-            const double cost = kChunkCost[want_adaptive ? 1 : 0][c] * ceil_div(s.M, kBwdCfgRows[c] * kBwdCfgWaves[c]);
-            if (c == 0 || cost < best) { best = cost; cfg = c; }
+            const double cost = kChunkCost[pl.want_adaptive ? 1 : 0][c] * ceil_div(s.M, kBwdCfgRows[c] * kBwdCfgWaves[c]);
+            if (c == 0 || cost < best) { best = cost; pl.cfg = c; }
         }
     }
-    const int rows_per_wg = small ? kBwdSmallRows : kBwdCfgRows[cfg] * kBwdCfgWaves[cfg];
+    pl.rows_per_wg = small ? kBwdSmallRows : kBwdCfgRows[pl.cfg] * kBwdCfgWaves[pl.cfg];
+    return pl;
+}
+
+size_t norm_backward_scratch_bytes(const Geom& s, float p) {
+    const BwdPlan pl = plan_backward(s, p);
+    const size_t mpad = (size_t)ceil_div(s.M, pl.rows_per_wg) * pl.rows_per_wg;
+    return (size_t)s.COg * s.G * mpad * sizeof(float) * (pl.ip == -2 ? 2 : 1);
+}
+
+int launch_norm_backward(const float* gout, const float* x, const float* w, const float* out, const Geom& s, float* gx,
+                         float* gw, float p, hipStream_t st) {
+    const float q = p - 1.0f;
+    const BwdPlan pl = plan_backward(s, p);
+    const int ip = pl.ip, cfg = pl.cfg;
+    const bool want_adaptive = pl.want_adaptive;
+    const int rows_per_wg = pl.rows_per_wg;
 
     BwdParams P{};
     P.s = s;

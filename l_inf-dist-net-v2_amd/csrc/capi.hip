@@ -20,6 +20,12 @@ bool hip_failed(hipError_t e) {
     return true;
 }
 
+int hip_status(hipError_t e) {
+    if (!hip_failed(e)) return NDIST_OK;
+    if (e == hipErrorStreamCaptureUnsupported) return NDIST_ERR_CAPTURE;
+    return NDIST_ERR_HIP;
+}
+
 const DeviceInfo& device_info() {
     constexpr int kMaxDev = 64;
     static DeviceInfo cache[kMaxDev];
@@ -52,6 +58,11 @@ static std::mutex g_ev_mu;
 
 KernelTimer::KernelTimer(hipStream_t st) : stream(st), active(g_profiling.load(std::memory_order_relaxed) != 0) {
     if (!active) return;
+    // no event records into a graph under capture
+    if (stream_is_capturing(st)) {
+        active = false;
+        return;
+    }
     if (g_timer_depth++ > 0) return;
     std::lock_guard<std::mutex> lock(g_ev_mu);
     if (g_ev_start == nullptr) {
@@ -125,6 +136,7 @@ const char* ndist_status_string(int status) {
         case NDIST_ERR_BAD_P: return "p must be positive and finite";
         case NDIST_ERR_HIP: return "a HIP runtime call failed";
         case NDIST_ERR_NO_DEVICE: return "no usable HIP device";
+        case NDIST_ERR_CAPTURE: return "the stream is being captured into a graph and this call needs temporary device memory";
         default: return "unknown status";
     }
 }
@@ -136,6 +148,13 @@ void ndist_set_profiling(int enable) { g_profiling.store(enable ? 1 : 0); }
 void ndist_set_skip_mode(int skip, int bounds) { set_skip_mode(skip, bounds); }
 
 int ndist_release_scratch(void) { return scratch_release_all(); }
+
+void ndist_scratch_counters(long* mallocs, long* frees) {
+    long m = 0, f = 0;
+    scratch_counters(&m, &f);
+    if (mallocs != nullptr) *mallocs = m;
+    if (frees != nullptr) *frees = f;
+}
 
 int ndist_last_kernel_ms(float* ms) {
     if (ms == nullptr) return NDIST_ERR_NULL_POINTER;

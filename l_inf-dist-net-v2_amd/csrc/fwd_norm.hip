@@ -723,7 +723,10 @@ int launch_norm_forward(const float* x, const float* w, const float* max_in, con
         P.thr = exp2f(-32.0f / p);
         P.inv_thr = 1.0f / P.thr;
         float* scratch = nullptr;  // probe scratch, then the seeds of the skipping operator (values, indices)
-        NDIST_HIP_TRY(scratch_alloc((void**)&scratch, (kProbeScratchFloats + seed_scratch_floats(s)) * sizeof(float), st));
+        if (scratch_alloc((void**)&scratch, (kProbeScratchFloats + seed_scratch_floats(s)) * sizeof(float), st) != hipSuccess) {
+            (void)hipGetLastError();  // no scratch (out of memory, or a stream under capture): the plain kernel needs none
+            return launch_fwd<OpNormalized<false>, CfgWideT, CfgMid, CfgSmall>(P, st);
+        }
         int* gate = reinterpret_cast<int*>(scratch);
         int rc = launch_norm_probe_steps(x, w, s, P.thr, scratch, st);
         P.gate = gate;

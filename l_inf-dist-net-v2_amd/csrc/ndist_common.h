@@ -53,6 +53,9 @@ const DeviceInfo& device_info();
 
 // Records a failing HIP call for ndist_last_hip_error(); returns true when `e` is an error.
 bool hip_failed(hipError_t e);
+// The same, as an ndist_status value: 0 for success, NDIST_ERR_CAPTURE when scratch was refused because the stream
+// is being captured, else NDIST_ERR_HIP.
+int hip_status(hipError_t e);
 
 // Optional timing of the dominant kernel of an entry point (see ndist_set_profiling): when enabled, the launcher
 // brackets that one kernel with two events on the launch stream; ndist_last_kernel_ms() reads them back.
@@ -67,10 +70,16 @@ struct KernelTimer {
 // same shape as hipMallocAsync / hipFreeAsync, but without their wait for the stream's queued work, and without any
 // allocation once the arena has grown to the largest request of its stream.  Releases go in reverse order of the
 // requests; every request of a call must be released before the call returns.
+// A request made while `st` is being captured into a graph fails with hipErrorStreamCaptureUnsupported before
+// anything is allocated or launched.
 hipError_t scratch_alloc(void** out, size_t bytes, hipStream_t st);
 hipError_t scratch_free(void* p, hipStream_t st);
 // Frees the memory of every arena no call is using (waits for the device).
 int scratch_release_all();
+// hipMalloc / hipFree calls made on behalf of the arenas since the library was loaded
+void scratch_counters(long* mallocs, long* frees);
+// true while `st` is being captured into a graph (or its state cannot be queried)
+bool stream_is_capturing(hipStream_t st);
 
 // Seeds and k-tile bounds for the forward operators that skip whole k-tiles (fully-connected layout, HW == 1).
 //   seed    [M][COg*G] as the output: for every output, the larger of the two pairs |x - w| at the k where its x row
@@ -93,9 +102,9 @@ size_t seed_scratch_floats(const Geom& s);
 int launch_seeds(const float* x, const float* w, const Geom& s, float* base, const int* gate, int gate_limit,
                  hipStream_t st, SeedBuffers* out, const float* x2 = nullptr);
 
-#define NDIST_HIP_TRY(expr)                          \
-    do {                                             \
-        if (::ndist::hip_failed((expr))) return 4;   \
+#define NDIST_HIP_TRY(expr)                                        \
+    do {                                                           \
+        if (int rc_try_ = ::ndist::hip_status((expr))) return rc_try_; \
     } while (0)
 
 // geometry of the patch extraction [B, C, H, W] -> [B, C*kh*kw, OH*OW]
@@ -192,6 +201,8 @@ int launch_norm_forward(const float* x, const float* w, const float* max_in, con
                         hipStream_t st);
 int launch_norm_backward(const float* gout, const float* x, const float* w, const float* out, const Geom& s,
                          float* gx, float* gw, float p, hipStream_t st);
+// bytes of scratch launch_norm_backward cannot do without (the factor array); everything else it asks for is optional
+size_t norm_backward_scratch_bytes(const Geom& s, float p);
 // With a patch geometry the input gradients are images [B, C, H, W] (the adjoint of the patch extraction is applied
 // on the fly); the launcher returns -1 when the geometry does not fit its kernels and nothing was launched.
 int launch_inf_backward(const float* gout, const int32_t* pos, const Geom& s, float* gx, float* gw, hipStream_t st,

@@ -11,6 +11,7 @@
 // threads that call on the same stream at the same time get two arenas.  Within a call the allocations are
 // released in reverse order (a stack).  The blocking hipMalloc / hipFree appear only while an arena is still
 // growing towards the largest request of its stream, i.e. in the first calls of each shape.
+#include <atomic>
 #include <mutex>
 #include <vector>
 
@@ -21,6 +22,9 @@ namespace ndist {
 namespace {
 
 constexpr size_t kAlign = 256;
+
+std::atomic<long> g_mallocs{0}, g_frees{0};  // hipMalloc / hipFree calls made for the arenas (scratch_counters)
+
 
 struct Block {
     char* base;
@@ -48,7 +52,10 @@ thread_local Current t_cur;
 size_t aligned(size_t n) { return (n + kAlign - 1) / kAlign * kAlign; }
 
 void free_blocks(Arena* a) {
-    for (Block& b : a->blocks) (void)hipFree(b.base);  // hipFree waits for the device: nothing still reads the block
+    for (Block& b : a->blocks) {
+        (void)hipFree(b.base);  // hipFree waits for the device: nothing still reads the block
+        g_frees++;
+    }
     a->blocks.clear();
 }
 
@@ -73,8 +80,12 @@ Arena* acquire(hipStream_t st) {
         free_blocks(a);
         char* p = nullptr;
         const size_t want = aligned(a->high + a->high / 4);
-        if (hipMalloc((void**)&p, want) == hipSuccess) a->blocks.push_back(Block{p, want, 0});
-        else (void)hipGetLastError();  // the blocks come back one request at a time
+        if (hipMalloc((void**)&p, want) == hipSuccess) {
+            a->blocks.push_back(Block{p, want, 0});
+            g_mallocs++;
+        } else {
+            (void)hipGetLastError();  // the blocks come back one request at a time
+        }
     }
     a->live = 0;
     a->cur = 0;
@@ -89,8 +100,27 @@ void release(Arena* a) {
 
 }  // namespace
 
+bool stream_is_capturing(hipStream_t st) {
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    // an error here (e.g. the legacy stream while another stream captures globally) also means "do not touch it"
+    if (hipStreamIsCapturing(st, &cs) != hipSuccess) {
+        (void)hipGetLastError();
+        return true;
+    }
+    return cs != hipStreamCaptureStatusNone;
+}
+
+void scratch_counters(long* mallocs, long* frees) {
+    *mallocs = g_mallocs.load();
+    *frees = g_frees.load();
+}
+
 hipError_t scratch_alloc(void** out, size_t bytes, hipStream_t st) {
     *out = nullptr;
+    // A stream that is being captured into a graph must see neither an allocation (hipMalloc is not permitted
+    // during a capture, and a later hipFree of the block would leave the graph with a dangling address) nor a
+    // block address that only this call's arena guarantees: calls that need scratch refuse to run under capture.
+    if (stream_is_capturing(st)) return hipErrorStreamCaptureUnsupported;
     if (t_cur.arena != nullptr && t_cur.arena->stream != st) {
         // a call that failed between a request and its release left its arena attached to this thread
         release(t_cur.arena);
@@ -111,6 +141,7 @@ hipError_t scratch_alloc(void** out, size_t bytes, hipStream_t st) {
             if (a->live == 0) { release(a); t_cur.arena = nullptr; }
             return e;
         }
+        g_mallocs++;
         a->blocks.push_back(Block{p, need, 0});
         blk = &a->blocks.back();
     }
