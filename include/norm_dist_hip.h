@@ -42,8 +42,9 @@ enum ndist_status {
     NDIST_ERR_BAD_P = 3,          /* p <= 0, NaN, or infinite where a finite p is required */
     NDIST_ERR_HIP = 4,            /* a HIP runtime call failed; see ndist_last_hip_error() */
     NDIST_ERR_NO_DEVICE = 5,      /* no HIP device is usable */
-    NDIST_ERR_CAPTURE = 6         /* the stream is being captured into a HIP graph and the call needs temporary device
+    NDIST_ERR_CAPTURE = 6,        /* the stream is being captured into a HIP graph and the call needs temporary device
                                      memory from the library's arenas: nothing was allocated or launched */
+    NDIST_ERR_TOO_LARGE = 7       /* ndist_*_noalloc: the problem needs more scratch than the fixed array holds */
 };
 
 /* Library version (major * 10000 + minor * 100 + patch). */
@@ -79,7 +80,8 @@ int ndist_release_scratch(void);
 void ndist_scratch_counters(long* mallocs, long* frees);
 /* HIP graphs: an entry point that would take arena scratch returns NDIST_ERR_CAPTURE when `stream` is being captured
  * (before it allocates or launches anything): a captured graph must not hold addresses of memory a later call may
- * free.  Entry points and shapes that need no scratch can be captured. */
+ * free.  Entry points and shapes that need no scratch can be captured; ndist_norm_dist_backward_input_weight_noalloc
+ * never takes arena scratch. */
 
 /* ---- finite p: replaces template struct norm_dist<ip> (core/cuda/norm_dist.h:4-14) ------------------- */
 
@@ -103,6 +105,23 @@ int ndist_norm_dist_backward_input(const float* grad_output, const float* input,
 int ndist_norm_dist_backward_input_weight(const float* grad_output, const float* input, const float* weight,
                                           const float* output, int B, int CO, int CI, int G, int HW,
                                           float* grad_input, float* grad_weight, float p, ndist_stream_t stream);
+
+/* No counterpart in the reference.  For callers that cannot allocate device memory at the time of the call (code
+ * under HIP graph capture, serving loops and harnesses that forbid hipMalloc): the same computation and arguments as
+ * ndist_norm_dist_backward_input_weight, but every byte of temporary device memory (the per-(row, output) factor
+ * array of the fused kernel, and the few words of the large-exponent probes) comes from one fixed array of
+ * ndist_noalloc_scratch_bytes() = 24 MiB that is part of the library's code object and that every GPU holds until
+ * the process ends.  The call makes no hipMalloc / hipFree / event creation, whatever the arenas hold.  Problems whose factor
+ * array, G*CO/G x (B*HW rounded up to the kernel's row chunk) floats (twice that for 1 < p < 2), exceeds the array
+ * return NDIST_ERR_TOO_LARGE before anything is launched (B*HW x CO up to 6.29 M, e.g. 512 x 5120 twice over); the
+ * conv layout runs without the transposed copies of the allocating entry point when they do not fit.  All calls on
+ * one GPU share that GPU's array: calls that overlap in time on one device (two streams, two threads) race; calls
+ * queued on one stream do not.  Results are those of ndist_norm_dist_backward_input_weight. */
+int ndist_norm_dist_backward_input_weight_noalloc(const float* grad_output, const float* input, const float* weight,
+                                                  const float* output, int B, int CO, int CI, int G, int HW,
+                                                  float* grad_input, float* grad_weight, float p,
+                                                  ndist_stream_t stream);
+size_t ndist_noalloc_scratch_bytes(void);
 
 /* ---- p = infinity: replaces struct inf_dist (core/cuda/norm_dist.h:16-25) ---------------------------- */
 

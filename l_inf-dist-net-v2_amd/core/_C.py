@@ -47,12 +47,15 @@ _lib.ndist_last_kernel_ms.argtypes = [ctypes.POINTER(ctypes.c_float)]
 _lib.ndist_last_kernel_ms.restype = ctypes.c_int
 _lib.ndist_scratch_counters.argtypes = [ctypes.POINTER(ctypes.c_long), ctypes.POINTER(ctypes.c_long)]
 _lib.ndist_scratch_counters.restype = None
+_lib.ndist_noalloc_scratch_bytes.argtypes = []
+_lib.ndist_noalloc_scratch_bytes.restype = ctypes.c_size_t
 
 _DIMS = (_I, _I, _I, _I, _I)
 _norm_fwd = _sig("ndist_norm_dist_forward", _P, _P, *_DIMS, _P, _F, _P)
 _norm_fwd_max = _sig("ndist_norm_dist_forward_with_max", _P, _P, _P, *_DIMS, _P, _F, _P)
 _norm_bwd_x = _sig("ndist_norm_dist_backward_input", _P, _P, _P, _P, *_DIMS, _P, _F, _P)
 _norm_bwd_xw = _sig("ndist_norm_dist_backward_input_weight", _P, _P, _P, _P, *_DIMS, _P, _P, _F, _P)
+_norm_bwd_xw_noalloc = _sig("ndist_norm_dist_backward_input_weight_noalloc", _P, _P, _P, _P, *_DIMS, _P, _P, _F, _P)
 _inf_fwd_ng = _sig("ndist_inf_dist_forward_nograd", _P, _P, *_DIMS, _P, _P)
 _inf_fwd = _sig("ndist_inf_dist_forward", _P, _P, *_DIMS, _P, _P, _P)
 _inf_bwd_x = _sig("ndist_inf_dist_backward_input", _P, _P, *_DIMS, _P, _P)
@@ -75,6 +78,7 @@ _conv_bnd_bwd_xw = _sig("ndist_conv_bound_inf_dist_backward_input_weight", _P, _
 
 # status codes of the library (include/norm_dist_hip.h)
 ERR_CAPTURE = 6
+ERR_TOO_LARGE = 7
 
 
 class NormDistError(RuntimeError):
@@ -94,6 +98,11 @@ def scratch_counters():
     m, f = ctypes.c_long(0), ctypes.c_long(0)
     _lib.ndist_scratch_counters(ctypes.byref(m), ctypes.byref(f))
     return m.value, f.value
+
+
+def noalloc_scratch_bytes():
+    """Size of the fixed scratch array behind norm_dist_backward_input_weight_noalloc."""
+    return int(_lib.ndist_noalloc_scratch_bytes())
 
 
 def set_profiling(enable):
@@ -181,6 +190,17 @@ def norm_dist_backward_input_weight(grad_output, input, weight, output, grad_inp
     B, CO, CI, HW = grad_output.size(0), output.size(1), input.size(1), input.size(2)
     _run(_norm_bwd_xw, dev, _p(grad_output), _p(input), _p(weight), _p(output), B, CO, CI, G, HW,
          _p(grad_input), _p(grad_weight), p)
+
+
+def norm_dist_backward_input_weight_noalloc(grad_output, input, weight, output, grad_input, grad_weight, G, p,
+                                            stream=None):
+    """norm_dist_backward_input_weight without any allocation inside the library (scratch from a fixed device array);
+    no counterpart in the reference.  `stream`: a raw hipStream_t to launch on instead of torch's current stream."""
+    dev = _check({}, grad_output=grad_output, input=input, weight=weight, output=output, grad_input=grad_input,
+                 grad_weight=grad_weight)
+    B, CO, CI, HW = grad_output.size(0), output.size(1), input.size(1), input.size(2)
+    _run(_norm_bwd_xw_noalloc, dev, _p(grad_output), _p(input), _p(weight), _p(output), B, CO, CI, G, HW,
+         _p(grad_input), _p(grad_weight), p, stream=stream)
 
 
 def inf_dist_forward(input, weight, output, pos, G):

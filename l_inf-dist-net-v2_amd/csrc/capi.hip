@@ -23,6 +23,7 @@ bool hip_failed(hipError_t e) {
 int hip_status(hipError_t e) {
     if (!hip_failed(e)) return NDIST_OK;
     if (e == hipErrorStreamCaptureUnsupported) return NDIST_ERR_CAPTURE;
+    if (e == hipErrorOutOfMemory && static_scratch_active()) return NDIST_ERR_TOO_LARGE;
     return NDIST_ERR_HIP;
 }
 
@@ -58,8 +59,8 @@ static std::mutex g_ev_mu;
 
 KernelTimer::KernelTimer(hipStream_t st) : stream(st), active(g_profiling.load(std::memory_order_relaxed) != 0) {
     if (!active) return;
-    // no event records into a graph under capture
-    if (stream_is_capturing(st)) {
+    // no event records into a graph under capture, and nothing that allocates inside the no-allocation entry point
+    if (static_scratch_active() || stream_is_capturing(st)) {
         active = false;
         return;
     }
@@ -137,6 +138,7 @@ const char* ndist_status_string(int status) {
         case NDIST_ERR_HIP: return "a HIP runtime call failed";
         case NDIST_ERR_NO_DEVICE: return "no usable HIP device";
         case NDIST_ERR_CAPTURE: return "the stream is being captured into a graph and this call needs temporary device memory";
+        case NDIST_ERR_TOO_LARGE: return "the problem needs more temporary device memory than the fixed scratch array holds";
         default: return "unknown status";
     }
 }
@@ -155,6 +157,8 @@ void ndist_scratch_counters(long* mallocs, long* frees) {
     if (mallocs != nullptr) *mallocs = m;
     if (frees != nullptr) *frees = f;
 }
+
+size_t ndist_noalloc_scratch_bytes(void) { return kStaticScratchBytes; }
 
 int ndist_last_kernel_ms(float* ms) {
     if (ms == nullptr) return NDIST_ERR_NULL_POINTER;
@@ -202,6 +206,22 @@ int ndist_norm_dist_backward_input_weight(const float* grad_output, const float*
     if (!finite_positive(p)) return NDIST_ERR_BAD_P;
     Geom s;
     if (int rc = make_geom(B, CO, CI, G, HW, &s)) return rc;
+    return launch_norm_backward(grad_output, input, weight, output, s, grad_input, grad_weight, p, (hipStream_t)stream);
+}
+
+int ndist_norm_dist_backward_input_weight_noalloc(const float* grad_output, const float* input, const float* weight,
+                                                  const float* output, int B, int CO, int CI, int G, int HW,
+                                                  float* grad_input, float* grad_weight, float p,
+                                                  ndist_stream_t stream) {
+    NDIST_REQUIRE(grad_output); NDIST_REQUIRE(input); NDIST_REQUIRE(weight); NDIST_REQUIRE(output);
+    NDIST_REQUIRE(grad_input); NDIST_REQUIRE(grad_weight);
+    if (!finite_positive(p)) return NDIST_ERR_BAD_P;
+    Geom s;
+    if (int rc = make_geom(B, CO, CI, G, HW, &s)) return rc;
+    // the factor array is the one piece of scratch the kernels cannot do without: refuse before anything is launched
+    if (norm_backward_scratch_bytes(s, p) > kStaticScratchBytes) return NDIST_ERR_TOO_LARGE;
+    StaticScratchScope scope;  // scratch_alloc serves from the fixed array while this lives; looks its address up once
+    if (int rc = hip_status(scope.status)) return rc;
     return launch_norm_backward(grad_output, input, weight, output, s, grad_input, grad_weight, p, (hipStream_t)stream);
 }
 

@@ -54,7 +54,7 @@ const DeviceInfo& device_info();
 // Records a failing HIP call for ndist_last_hip_error(); returns true when `e` is an error.
 bool hip_failed(hipError_t e);
 // The same, as an ndist_status value: 0 for success, NDIST_ERR_CAPTURE when scratch was refused because the stream
-// is being captured, else NDIST_ERR_HIP.
+// is being captured, NDIST_ERR_TOO_LARGE when the fixed scratch array is too small, else NDIST_ERR_HIP.
 int hip_status(hipError_t e);
 
 // Optional timing of the dominant kernel of an entry point (see ndist_set_profiling): when enabled, the launcher
@@ -80,6 +80,23 @@ int scratch_release_all();
 void scratch_counters(long* mallocs, long* frees);
 // true while `st` is being captured into a graph (or its state cannot be queried)
 bool stream_is_capturing(hipStream_t st);
+
+// Scratch without any allocation: a fixed array of kStaticScratchBytes in device memory, one copy per device.  While
+// a StaticScratchScope lives on the calling thread, scratch_alloc serves from that array (stack-ordered, failing
+// with hipErrorOutOfMemory beyond its size) and calls no allocator; calls that overlap on one device share the
+// array and race.
+constexpr size_t kStaticScratchBytes = 24u << 20;
+struct StaticScratchScope {
+    StaticScratchScope();
+    ~StaticScratchScope();
+    StaticScratchScope(const StaticScratchScope&) = delete;
+    StaticScratchScope& operator=(const StaticScratchScope&) = delete;
+    hipError_t status;  // of the one-time address lookup
+    char* base;         // device address of this device's copy of the array
+    size_t used;
+    int live;
+};
+bool static_scratch_active();
 
 // Seeds and k-tile bounds for the forward operators that skip whole k-tiles (fully-connected layout, HW == 1).
 //   seed    [M][COg*G] as the output: for every output, the larger of the two pairs |x - w| at the k where its x row

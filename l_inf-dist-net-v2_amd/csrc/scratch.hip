@@ -11,6 +11,10 @@
 // threads that call on the same stream at the same time get two arenas.  Within a call the allocations are
 // released in reverse order (a stack).  The blocking hipMalloc / hipFree appear only while an arena is still
 // growing towards the largest request of its stream, i.e. in the first calls of each shape.
+//
+// Callers that cannot allocate at all use the entry point that takes its scratch from a fixed array in device
+// memory instead (static scratch, below): while a StaticScratchScope is alive on the calling thread, scratch_alloc
+// hands out pieces of that array and never touches the arenas or the HIP allocator.
 #include <atomic>
 #include <mutex>
 #include <vector>
@@ -19,12 +23,18 @@
 
 namespace ndist {
 
+// Scratch of the entry point that allocates nothing: one array per device, part of the code object, alive until the
+// process ends.  Host code never uses the array's name as an address: the device address is looked up once per
+// device with hipGetSymbolAddress (static_scratch_base) and passed to the kernels like any other buffer.
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace {
 
 constexpr size_t kAlign = 256;
 
 std::atomic<long> g_mallocs{0}, g_frees{0};  // hipMalloc / hipFree calls made for the arenas (scratch_counters)
 
+thread_local StaticScratchScope* t_static = nullptr;  // lives on the stack of the entry point
 
 struct Block {
     char* base;
@@ -110,6 +120,36 @@ bool stream_is_capturing(hipStream_t st) {
     return cs != hipStreamCaptureStatusNone;
 }
 
+hipError_t static_scratch_base(char** out) {
+    constexpr int kMaxDev = 64;
+    static char* base[kMaxDev] = {};
+    static std::mutex mu;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDev) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(mu);
+    if (base[dev] == nullptr) {
+        // once per device, with that device current: every device holds its own copy of the array
+        char* ptr = nullptr;
+        e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (ptr == nullptr) return hipErrorInvalidSymbol;
+        base[dev] = ptr;
+    }
+    *out = base[dev];
+    return hipSuccess;
+}
+
+StaticScratchScope::StaticScratchScope() : status(hipSuccess), base(nullptr), used(0), live(0) {
+    status = static_scratch_base(&base);
+    if (status == hipSuccess) t_static = this;
+}
+StaticScratchScope::~StaticScratchScope() {
+    if (t_static == this) t_static = nullptr;
+}
+bool static_scratch_active() { return t_static != nullptr; }
+
 void scratch_counters(long* mallocs, long* frees) {
     *mallocs = g_mallocs.load();
     *frees = g_frees.load();
@@ -117,6 +157,15 @@ void scratch_counters(long* mallocs, long* frees) {
 
 hipError_t scratch_alloc(void** out, size_t bytes, hipStream_t st) {
     *out = nullptr;
+    if (t_static != nullptr) {
+        // pieces of the fixed array, stack-ordered like the arena's; no allocation, no query of the stream
+        const size_t need = aligned(bytes == 0 ? 1 : bytes);
+        if (need > kStaticScratchBytes - t_static->used) return hipErrorOutOfMemory;
+        *out = t_static->base + t_static->used;
+        t_static->used += need;
+        t_static->live++;
+        return hipSuccess;
+    }
     // A stream that is being captured into a graph must see neither an allocation (hipMalloc is not permitted
     // during a capture, and a later hipFree of the block would leave the graph with a dangling address) nor a
     // block address that only this call's arena guarantees: calls that need scratch refuse to run under capture.
@@ -154,6 +203,14 @@ hipError_t scratch_alloc(void** out, size_t bytes, hipStream_t st) {
 }
 
 hipError_t scratch_free(void* p, hipStream_t) {
+    if (t_static != nullptr) {
+        char* c = static_cast<char*>(p);
+        if (p == nullptr || t_static->live == 0 || c < t_static->base || c >= t_static->base + t_static->used)
+            return hipErrorInvalidValue;
+        t_static->used = (size_t)(c - t_static->base);
+        t_static->live--;
+        return hipSuccess;
+    }
     Arena* a = t_cur.arena;
     if (p == nullptr || a == nullptr || a->live == 0) return hipErrorInvalidValue;
     // stack order: p is the most recent allocation still alive, at the end of the last block in use
