@@ -34,6 +34,15 @@ def test_forward_vs_reference_formula(G, HW):
     np.testing.assert_array_equal(iu, mx.argmax(2))
     branch = (t1 > t2).reshape(B, CO, CIg, HW)  # flag set iff not (t1 <= t2)
     np.testing.assert_array_equal(su, np.take_along_axis(branch, mx.argmax(2)[:, :, None, :], 2)[:, :, 0, :])
+    # lower bound: first occurrence of the minimum of min(t1, t2) and the branch active there (reference:
+    # core/cuda/bound_inf_dist_cuda.cu:203-213); outputs that stayed at the floor carry the "no gradient" code
+    mn = np.minimum(t1, t2).reshape(B, CO, CIg, HW)
+    il, sl = O.decode_pos(pl)
+    moved = yl > np.float32(1e-10)
+    assert moved.any()
+    np.testing.assert_array_equal(il[moved], mn.argmin(2)[moved])
+    np.testing.assert_array_equal(sl[moved], np.take_along_axis(branch, mn.argmin(2)[:, :, None, :], 2)[:, :, 0, :][moved])
+    np.testing.assert_array_equal(pl.view(np.uint32)[~moved], np.uint32(0xffffffff))
     yl2, yu2, n1, n2 = O.bound_inf_dist_forward(xl, xu, w, G, with_pos=False)
     assert n1 is None and n2 is None
     np.testing.assert_array_equal(yl, yl2)
