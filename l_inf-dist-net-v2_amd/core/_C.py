@@ -1,13 +1,19 @@
 """Binding of libnorm_dist_hip.so: the twelve kernel entry points under the names, argument orders and checks of the
 reference's extension module (core/cuda/norm_dist.cpp:40-204), taking torch tensors.
 
-Importing this module fails loudly when the library has not been built: there is no fallback implementation.
+Two routes lead to the same C ABI.  The PyTorch C++ extension `norm_dist_hip_ext` (csrc/binding/norm_dist_ext.cpp,
+built next to the library) is used when it is there: it validates the tensors, makes their device current and
+launches on PyTorch's current stream from compiled code.  Without it (or with NORM_DIST_BINDING=ctypes) the same
+calls go through ctypes from this file, with the same checks written in Python.  Either way, importing this module
+fails loudly when the library itself has not been built: there is no fallback implementation of the kernels.
 Each call validates its tensors the way the reference's CHECK_INPUT does (device + contiguity, core/cuda/norm_dist.cpp:8-10)
 plus dtype, derives (B, CO, CI, HW) exactly as the reference does, and launches on torch's current stream of the
 tensors' device.
 """
 import ctypes
 import os
+import re
+import sys
 
 import torch
 
@@ -20,6 +26,17 @@ if not os.path.exists(_LIB_PATH):
         (_LIB_PATH, os.path.join(os.path.dirname(os.path.dirname(_LIB_PATH)), "csrc")))
 _lib = ctypes.CDLL(_LIB_PATH)
 LIBRARY_PATH = _LIB_PATH
+
+# The compiled binding, when it has been built (it links against the library above, same directory).
+_ext = None
+EXTENSION_PATH = os.path.join(os.path.dirname(_LIB_PATH), "norm_dist_hip_ext.so")
+if os.environ.get("NORM_DIST_BINDING", "ext") != "ctypes" and os.path.exists(EXTENSION_PATH):
+    import importlib.util
+    _spec = importlib.util.spec_from_file_location("norm_dist_hip_ext", EXTENSION_PATH)
+    _ext = importlib.util.module_from_spec(_spec)
+    _spec.loader.exec_module(_ext)
+    sys.modules.setdefault("norm_dist_hip_ext", _ext)
+BINDING = "ext" if _ext is not None else "ctypes"
 
 _P = ctypes.c_void_p
 _I = ctypes.c_int
@@ -163,28 +180,54 @@ def _p(t):
     return t.data_ptr()
 
 
+_STATUS_RE = re.compile(r"\(status (\d+),")
+
+
+def _ext_call(fn, *args):
+    """Call into the compiled binding; its errors carry the library's status code in their text."""
+    try:
+        fn(*args)
+    except RuntimeError as e:
+        m = _STATUS_RE.search(str(e))
+        if m:
+            raise NormDistError(str(e).split("\n")[0], int(m.group(1))) from None
+        raise
+
+
+def _geo8(geo):
+    return list(geo[4:12])
+
+
 _INT = {"pos": torch.int32, "posL": torch.int32, "posU": torch.int32}
 
 
 def norm_dist_forward(input, weight, output, G, p):
+    if _ext is not None:
+        return _ext_call(_ext.norm_dist_forward, input, weight, output, G, p)
     dev = _check({}, input=input, weight=weight, output=output)
     B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
     _run(_norm_fwd, dev, _p(input), _p(weight), B, CO, CI, G, HW, _p(output), p)
 
 
 def norm_dist_forward_with_max(input, weight, max_output, output, G, p):
+    if _ext is not None:
+        return _ext_call(_ext.norm_dist_forward_with_max, input, weight, max_output, output, G, p)
     dev = _check({}, input=input, weight=weight, max_output=max_output, output=output)
     B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
     _run(_norm_fwd_max, dev, _p(input), _p(weight), _p(max_output), B, CO, CI, G, HW, _p(output), p)
 
 
 def norm_dist_backward_input(grad_output, input, weight, output, grad_input, G, p):
+    if _ext is not None:
+        return _ext_call(_ext.norm_dist_backward_input, grad_output, input, weight, output, grad_input, G, p)
     dev = _check({}, grad_output=grad_output, input=input, weight=weight, output=output, grad_input=grad_input)
     B, CO, CI, HW = grad_output.size(0), output.size(1), input.size(1), input.size(2)
     _run(_norm_bwd_x, dev, _p(grad_output), _p(input), _p(weight), _p(output), B, CO, CI, G, HW, _p(grad_input), p)
 
 
 def norm_dist_backward_input_weight(grad_output, input, weight, output, grad_input, grad_weight, G, p):
+    if _ext is not None:
+        return _ext_call(_ext.norm_dist_backward_input_weight, grad_output, input, weight, output, grad_input, grad_weight, G, p)
     dev = _check({}, grad_output=grad_output, input=input, weight=weight, output=output, grad_input=grad_input,
                  grad_weight=grad_weight)
     B, CO, CI, HW = grad_output.size(0), output.size(1), input.size(1), input.size(2)
@@ -196,6 +239,9 @@ def norm_dist_backward_input_weight_noalloc(grad_output, input, weight, output, 
                                             stream=None):
     """norm_dist_backward_input_weight without any allocation inside the library (scratch from a fixed device array);
     no counterpart in the reference.  `stream`: a raw hipStream_t to launch on instead of torch's current stream."""
+    if _ext is not None and stream is None:
+        return _ext_call(_ext.norm_dist_backward_input_weight_noalloc, grad_output, input, weight, output, grad_input,
+                         grad_weight, G, p)
     dev = _check({}, grad_output=grad_output, input=input, weight=weight, output=output, grad_input=grad_input,
                  grad_weight=grad_weight)
     B, CO, CI, HW = grad_output.size(0), output.size(1), input.size(1), input.size(2)
@@ -204,36 +250,48 @@ def norm_dist_backward_input_weight_noalloc(grad_output, input, weight, output, 
 
 
 def inf_dist_forward(input, weight, output, pos, G):
+    if _ext is not None:
+        return _ext_call(_ext.inf_dist_forward, input, weight, output, pos, G)
     dev = _check(_INT, input=input, weight=weight, output=output, pos=pos)
     B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
     _run(_inf_fwd, dev, _p(input), _p(weight), B, CO, CI, G, HW, _p(output), _p(pos))
 
 
 def inf_dist_forward_nograd(input, weight, output, G):
+    if _ext is not None:
+        return _ext_call(_ext.inf_dist_forward_nograd, input, weight, output, G)
     dev = _check({}, input=input, weight=weight, output=output)
     B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
     _run(_inf_fwd_ng, dev, _p(input), _p(weight), B, CO, CI, G, HW, _p(output))
 
 
 def inf_dist_backward_input(grad_output, pos, grad_input, G):
+    if _ext is not None:
+        return _ext_call(_ext.inf_dist_backward_input, grad_output, pos, grad_input, G)
     dev = _check(_INT, grad_output=grad_output, pos=pos, grad_input=grad_input)
     B, CO, CI, HW = grad_output.size(0), grad_output.size(1), grad_input.size(1), grad_input.size(2)
     _run(_inf_bwd_x, dev, _p(grad_output), _p(pos), B, CO, CI, G, HW, _p(grad_input))
 
 
 def inf_dist_backward_input_weight(grad_output, pos, grad_input, grad_weight, G):
+    if _ext is not None:
+        return _ext_call(_ext.inf_dist_backward_input_weight, grad_output, pos, grad_input, grad_weight, G)
     dev = _check(_INT, grad_output=grad_output, pos=pos, grad_input=grad_input, grad_weight=grad_weight)
     B, CO, CI, HW = grad_output.size(0), grad_output.size(1), grad_weight.size(1) * G, grad_output.size(2)
     _run(_inf_bwd_xw, dev, _p(grad_output), _p(pos), B, CO, CI, G, HW, _p(grad_input), _p(grad_weight))
 
 
 def bound_inf_dist_forward_nograd(inputL, inputU, weight, outputL, outputU, G):
+    if _ext is not None:
+        return _ext_call(_ext.bound_inf_dist_forward_nograd, inputL, inputU, weight, outputL, outputU, G)
     dev = _check({}, inputL=inputL, inputU=inputU, weight=weight, outputL=outputL, outputU=outputU)
     B, CO, CI, HW = inputL.size(0), outputL.size(1), inputL.size(1), inputL.size(2)
     _run(_bnd_fwd_ng, dev, _p(inputL), _p(inputU), _p(weight), B, CO, CI, G, HW, _p(outputL), _p(outputU))
 
 
 def bound_inf_dist_forward(inputL, inputU, weight, outputL, outputU, posL, posU, G):
+    if _ext is not None:
+        return _ext_call(_ext.bound_inf_dist_forward, inputL, inputU, weight, outputL, outputU, posL, posU, G)
     dev = _check(_INT, inputL=inputL, inputU=inputU, weight=weight, outputL=outputL, outputU=outputU,
                  posL=posL, posU=posU)
     B, CO, CI, HW = inputL.size(0), outputL.size(1), inputL.size(1), inputL.size(2)
@@ -242,6 +300,8 @@ def bound_inf_dist_forward(inputL, inputU, weight, outputL, outputU, posL, posU,
 
 
 def bound_inf_dist_backward_input(grad_outputL, grad_outputU, posL, posU, grad_inputL, grad_inputU, G):
+    if _ext is not None:
+        return _ext_call(_ext.bound_inf_dist_backward_input, grad_outputL, grad_outputU, posL, posU, grad_inputL, grad_inputU, G)
     dev = _check(_INT, grad_outputL=grad_outputL, grad_outputU=grad_outputU, posL=posL, posU=posU,
                  grad_inputL=grad_inputL, grad_inputU=grad_inputU)
     B, CO, CI, HW = grad_outputL.size(0), grad_outputL.size(1), grad_inputL.size(1), grad_inputL.size(2)
@@ -251,6 +311,8 @@ def bound_inf_dist_backward_input(grad_outputL, grad_outputU, posL, posU, grad_i
 
 def bound_inf_dist_backward_input_weight(grad_outputL, grad_outputU, posL, posU, grad_inputL, grad_inputU,
                                          grad_weight, G):
+    if _ext is not None:
+        return _ext_call(_ext.bound_inf_dist_backward_input_weight, grad_outputL, grad_outputU, posL, posU, grad_inputL, grad_inputU, grad_weight, G)
     dev = _check(_INT, grad_outputL=grad_outputL, grad_outputU=grad_outputU, posL=posL, posU=posU,
                  grad_inputL=grad_inputL, grad_inputU=grad_inputU, grad_weight=grad_weight)
     B, CO, CI, HW = grad_outputL.size(0), grad_outputL.size(1), grad_weight.size(1) * G, grad_outputL.size(2)
@@ -278,6 +340,8 @@ def unfold_forward(input, output, kernel_size, dilation, padding, stride):
     geo, (OH, OW) = unfold_geometry(input.shape, kernel_size, dilation, padding, stride)
     if tuple(output.shape) != (geo[0], geo[1] * geo[4] * geo[5], OH * OW):
         raise RuntimeError("output has shape %s, expected %s" % (tuple(output.shape), (geo[0], geo[1] * geo[4] * geo[5], OH * OW)))
+    if _ext is not None:
+        return _ext_call(_ext.unfold_forward, input, output, _geo8(geo))
     _run(_unfold_fwd, dev, _p(input), *geo, _p(output))
 
 
@@ -287,6 +351,8 @@ def unfold_backward(grad_output, grad_input, kernel_size, dilation, padding, str
     geo, (OH, OW) = unfold_geometry(grad_input.shape, kernel_size, dilation, padding, stride)
     if tuple(grad_output.shape) != (geo[0], geo[1] * geo[4] * geo[5], OH * OW):
         raise RuntimeError("grad_output has shape %s, expected %s" % (tuple(grad_output.shape), (geo[0], geo[1] * geo[4] * geo[5], OH * OW)))
+    if _ext is not None:
+        return _ext_call(_ext.unfold_backward, grad_output, grad_input, _geo8(geo))
     _run(_unfold_bwd, dev, _p(grad_output), *geo, _p(grad_input))
 
 
@@ -306,6 +372,8 @@ def conv_inf_dist_forward_nograd(input, weight, output, G, kernel_size, dilation
     tensor is never written (the reference materialises it, core/modules/norm_dist.py:93-102)."""
     dev = _check({}, input=input, weight=weight, output=output)
     args = _conv_args(input, weight, output, G, kernel_size, dilation, padding, stride)
+    if _ext is not None:
+        return _ext_call(_ext.conv_inf_dist_forward_nograd, input, weight, output, G, list(args[6:14]))
     _run(_conv_inf_ng, dev, _p(input), _p(weight), *args, _p(output))
 
 
@@ -316,6 +384,9 @@ def conv_bound_inf_dist_forward_nograd(inputL, inputU, weight, outputL, outputU,
     if inputL.shape != inputU.shape or outputL.shape != outputU.shape:
         raise RuntimeError("lower and upper tensors must have the same shape")
     args = _conv_args(inputL, weight, outputL, G, kernel_size, dilation, padding, stride)
+    if _ext is not None:
+        return _ext_call(_ext.conv_bound_inf_dist_forward_nograd, inputL, inputU, weight, outputL, outputU, G,
+                         list(args[6:14]))
     _run(_conv_bnd_ng, dev, _p(inputL), _p(inputU), _p(weight), *args, _p(outputL), _p(outputU))
 
 
@@ -325,6 +396,8 @@ def conv_inf_dist_forward(input, weight, output, pos, G, kernel_size, dilation, 
     args = _conv_args(input, weight, output, G, kernel_size, dilation, padding, stride)
     if pos.shape != output.shape:
         raise RuntimeError("pos must have the shape of output")
+    if _ext is not None:
+        return _ext_call(_ext.conv_inf_dist_forward, input, weight, output, pos, G, list(args[6:14]))
     _run(_conv_inf_fwd, dev, _p(input), _p(weight), *args, _p(output), _p(pos))
 
 
@@ -335,6 +408,9 @@ def conv_bound_inf_dist_forward(inputL, inputU, weight, outputL, outputU, posL, 
     if inputL.shape != inputU.shape or not (outputL.shape == outputU.shape == posL.shape == posU.shape):
         raise RuntimeError("lower and upper tensors must have the same shape")
     args = _conv_args(inputL, weight, outputL, G, kernel_size, dilation, padding, stride)
+    if _ext is not None:
+        return _ext_call(_ext.conv_bound_inf_dist_forward, inputL, inputU, weight, outputL, outputU, posL, posU, G,
+                         list(args[6:14]))
     _run(_conv_bnd_fwd, dev, _p(inputL), _p(inputU), _p(weight), *args, _p(outputL), _p(outputU), _p(posL), _p(posU))
 
 
@@ -353,6 +429,8 @@ def conv_inf_dist_backward_input(grad_output, pos, grad_input, weight_shape, G, 
     """inf_dist_backward_input followed by the adjoint of the patch extraction: grad_input is [B, C, H, W]."""
     dev = _check(_INT, grad_output=grad_output, pos=pos, grad_input=grad_input)
     args = _conv_backward_args(grad_output, grad_input, weight_shape, G, kernel_size, dilation, padding, stride)
+    if _ext is not None:
+        return _ext_call(_ext.conv_inf_dist_backward_input, grad_output, pos, grad_input, args[4], G, list(args[6:14]))
     _run(_conv_inf_bwd_x, dev, _p(grad_output), _p(pos), *args, _p(grad_input))
 
 
@@ -360,6 +438,9 @@ def conv_inf_dist_backward_input_weight(grad_output, pos, grad_input, grad_weigh
                                         stride):
     dev = _check(_INT, grad_output=grad_output, pos=pos, grad_input=grad_input, grad_weight=grad_weight)
     args = _conv_backward_args(grad_output, grad_input, grad_weight.shape, G, kernel_size, dilation, padding, stride)
+    if _ext is not None:
+        return _ext_call(_ext.conv_inf_dist_backward_input_weight, grad_output, pos, grad_input, grad_weight, G,
+                         list(args[6:14]))
     _run(_conv_inf_bwd_xw, dev, _p(grad_output), _p(pos), *args, _p(grad_input), _p(grad_weight))
 
 
@@ -368,6 +449,9 @@ def conv_bound_inf_dist_backward_input(grad_outputL, grad_outputU, posL, posU, g
     dev = _check(_INT, grad_outputL=grad_outputL, grad_outputU=grad_outputU, posL=posL, posU=posU,
                  grad_inputL=grad_inputL, grad_inputU=grad_inputU)
     args = _conv_backward_args(grad_outputL, grad_inputL, weight_shape, G, kernel_size, dilation, padding, stride)
+    if _ext is not None:
+        return _ext_call(_ext.conv_bound_inf_dist_backward_input, grad_outputL, grad_outputU, posL, posU, grad_inputL,
+                         grad_inputU, args[4], G, list(args[6:14]))
     _run(_conv_bnd_bwd_x, dev, _p(grad_outputL), _p(grad_outputU), _p(posL), _p(posU), *args, _p(grad_inputL),
          _p(grad_inputU))
 
@@ -377,5 +461,8 @@ def conv_bound_inf_dist_backward_input_weight(grad_outputL, grad_outputU, posL, 
     dev = _check(_INT, grad_outputL=grad_outputL, grad_outputU=grad_outputU, posL=posL, posU=posU,
                  grad_inputL=grad_inputL, grad_inputU=grad_inputU, grad_weight=grad_weight)
     args = _conv_backward_args(grad_outputL, grad_inputL, grad_weight.shape, G, kernel_size, dilation, padding, stride)
+    if _ext is not None:
+        return _ext_call(_ext.conv_bound_inf_dist_backward_input_weight, grad_outputL, grad_outputU, posL, posU,
+                         grad_inputL, grad_inputU, grad_weight, G, list(args[6:14]))
     _run(_conv_bnd_bwd_xw, dev, _p(grad_outputL), _p(grad_outputU), _p(posL), _p(posU), *args, _p(grad_inputL),
          _p(grad_inputU), _p(grad_weight))

@@ -259,7 +259,7 @@ def test_conv_shape_fused_entry_points():
                  what="fused conv grad_weight")
     gx_only = torch.full_like(imd, float("nan"))
     _C.conv_inf_dist_backward_input(gd, pos, gx_only, w.shape, *geo)
-    assert rel_err(gx_only.cpu().numpy(), gx.cpu().numpy()) < 1e-6
+    assert_close(gx_only.cpu().numpy(), gx.cpu().numpy(), what="input-only entry point")  # LDS atomics: no fixed order
     del gx, gx_only
     # interval bounds on the images, eps = 8 / 255
     lo, up = imd - 8 / 255, imd + 8 / 255

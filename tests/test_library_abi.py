@@ -85,3 +85,21 @@ def test_unfold_geometry_and_validation():
     assert f(None, 1, 1, 4, 4, 3, 3, 1, 1, 1, 1, 1, 1, dummy, None) == 1
     assert f(dummy, 1, 1, 4, 4, 3, 3, 1, 1, 1, 1, 0, 1, dummy, None) == 2    # stride 0
     assert f(dummy, 1, 1, 2, 2, 5, 5, 1, 1, 0, 0, 1, 1, dummy, None) == 2    # window larger than the padded image
+
+
+def test_extension_module_exports_the_reference_names():
+    # the compiled PyTorch binding (csrc/binding/norm_dist_ext.cpp) imports without a GPU and carries the twelve
+    # functions of the reference's extension (core/cuda/norm_dist.cpp:191-204) plus this library's additions
+    from core import _C
+    assert _C.BINDING == "ext", "norm_dist_hip_ext.so has not been built"
+    E = _C._ext
+    for n in ["norm_dist_forward", "norm_dist_forward_with_max", "norm_dist_backward_input",
+              "norm_dist_backward_input_weight", "inf_dist_forward", "inf_dist_forward_nograd",
+              "inf_dist_backward_input", "inf_dist_backward_input_weight", "bound_inf_dist_forward",
+              "bound_inf_dist_forward_nograd", "bound_inf_dist_backward_input",
+              "bound_inf_dist_backward_input_weight", "norm_dist_backward_input_weight_noalloc", "unfold_forward",
+              "unfold_backward", "conv_inf_dist_forward", "conv_bound_inf_dist_backward_input_weight"]:
+        assert callable(getattr(E, n)), n
+    assert E.version() == _C.version()
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        E.norm_dist_forward(torch.zeros(2, 4, 1), torch.zeros(3, 4), torch.zeros(2, 3, 1), 1, 2.0)
