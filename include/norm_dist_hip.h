@@ -165,6 +165,26 @@ int ndist_bound_inf_dist_backward_input_weight(const float* grad_outputL, const 
                                                float* grad_inputL, float* grad_inputU, float* grad_weight,
                                                ndist_stream_t stream);
 
+/* ---- mean shift and bias of a distance layer ------------------------------------------------------------------
+ * The reference has no kernel of its own here: every layer follows the operator with MeanShift and a bias add
+ * written in torch primitives (core/modules/norm_dist.py:35-38, core/modules/basic_modules.py:121-132).  These two
+ * entry points do the same in two or three launches.  Tensors are [B, C, HW] like the operator's outputs.
+ *   forward:  mean[c] = training ? mean over (b, hw) of x : running_mean[c]   (0 when running_mean is NULL in evaluation)
+ *             y* = t* - mean[c] + bias1[c] + bias2[c]     for t* in {x, lower, upper} that are not NULL
+ *             training also writes mean_out[c] = mean[c] and running_mean[c] = (1 - momentum) running_mean[c] + momentum mean[c]
+ *             (running_mean may be NULL in training; bias1, bias2 may be NULL; x is required in training)
+ *   backward: colsum_out[c] = sum over (b, hw) of the given gradients (the gradient of either bias; may be NULL);
+ *             training: grad_x = grad_y - colsum / (B HW)  (grad_y required then; mean_scratch: [C] floats of the
+ *             caller's);  evaluation: grad_x is grad_y itself and is not written.
+ *             The gradients of lower and upper pass through unchanged and are not touched.
+ * Sums are taken in a fixed order: results repeat bit for bit. */
+int ndist_mean_shift_forward(const float* x, const float* lower, const float* upper, int B, int C, int HW, int training,
+                             float momentum, float* running_mean, const float* bias1, const float* bias2,
+                             float* mean_out, float* y, float* y_lower, float* y_upper, ndist_stream_t stream);
+int ndist_mean_shift_backward(const float* grad_y, const float* grad_y_lower, const float* grad_y_upper, int B, int C,
+                              int HW, int training, float* grad_x, float* colsum_out, float* mean_scratch,
+                              ndist_stream_t stream);
+
 /* ---- patch extraction for the convolutional layer -------------------------------------------------------------
  * The reference has no kernel of its own here: NormDistConv calls torch.nn.functional.unfold
  * (core/modules/norm_dist.py:93-102).  These two entry points replace that call and its autograd adjoint with one

@@ -81,6 +81,8 @@ _bnd_fwd_ng = _sig("ndist_bound_inf_dist_forward_nograd", _P, _P, _P, *_DIMS, _P
 _bnd_fwd = _sig("ndist_bound_inf_dist_forward", _P, _P, _P, *_DIMS, _P, _P, _P, _P, _P)
 _bnd_bwd_x = _sig("ndist_bound_inf_dist_backward_input", _P, _P, _P, _P, *_DIMS, _P, _P, _P)
 _bnd_bwd_xw = _sig("ndist_bound_inf_dist_backward_input_weight", _P, _P, _P, _P, *_DIMS, _P, _P, _P, _P)
+_ms_fwd = _sig("ndist_mean_shift_forward", _P, _P, _P, _I, _I, _I, _I, _F, _P, _P, _P, _P, _P, _P, _P, _P)
+_ms_bwd = _sig("ndist_mean_shift_backward", _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P)
 _unfold_fwd = _sig("ndist_unfold_forward", _P, *([_I] * 12), _P, _P)
 _unfold_bwd = _sig("ndist_unfold_backward", _P, *([_I] * 12), _P, _P)
 _conv_inf_ng = _sig("ndist_conv_inf_dist_forward_nograd", _P, _P, *([_I] * 14), _P, _P)
@@ -318,6 +320,44 @@ def bound_inf_dist_backward_input_weight(grad_outputL, grad_outputU, posL, posU,
     B, CO, CI, HW = grad_outputL.size(0), grad_outputL.size(1), grad_weight.size(1) * G, grad_outputL.size(2)
     _run(_bnd_bwd_xw, dev, _p(grad_outputL), _p(grad_outputU), _p(posL), _p(posU), B, CO, CI, G, HW,
          _p(grad_inputL), _p(grad_inputU), _p(grad_weight))
+
+
+def _po(t):
+    return None if t is None else t.data_ptr()
+
+
+def _check_some(**tensors):
+    return _check({}, **{k: v for k, v in tensors.items() if v is not None})
+
+
+def mean_shift_forward(x, lower, upper, training, momentum, running_mean, bias1, bias2, mean_out, y, y_lower, y_upper):
+    """Mean shift + bias of a distance layer in one call (no kernel of its own in the reference, which writes it in
+    torch primitives: core/modules/basic_modules.py:121-132, core/modules/norm_dist.py:35-38).  Tensors [B, C, HW];
+    absent ones are None.  y* = t* - mean[c] + bias1[c] + bias2[c] with mean the batch mean of x (training; also
+    written to mean_out and folded into running_mean) or running_mean (evaluation)."""
+    lead = x if x is not None else (lower if lower is not None else upper)
+    B, C, HW = lead.shape
+    if _ext is not None:
+        return _ext_call(_ext.mean_shift_forward, x, lower, upper, B, C, HW, bool(training), float(momentum), running_mean,
+                         bias1, bias2, mean_out, y, y_lower, y_upper)
+    dev = _check_some(x=x, lower=lower, upper=upper, running_mean=running_mean, bias1=bias1, bias2=bias2,
+                      mean_out=mean_out, y=y, y_lower=y_lower, y_upper=y_upper)
+    _run(_ms_fwd, dev, _po(x), _po(lower), _po(upper), B, C, HW, 1 if training else 0, float(momentum), _po(running_mean),
+         _po(bias1), _po(bias2), _po(mean_out), _po(y), _po(y_lower), _po(y_upper))
+
+
+def mean_shift_backward(grad_y, grad_y_lower, grad_y_upper, training, grad_x, colsum_out, mean_scratch):
+    """Backward of mean_shift_forward: colsum_out[c] = sum over (b, hw) of the given gradients (the bias gradient);
+    training: grad_x = grad_y - colsum / (B HW).  The bounds' gradients pass through unchanged."""
+    lead = grad_y if grad_y is not None else (grad_y_lower if grad_y_lower is not None else grad_y_upper)
+    B, C, HW = lead.shape
+    if _ext is not None:
+        return _ext_call(_ext.mean_shift_backward, grad_y, grad_y_lower, grad_y_upper, B, C, HW, bool(training), grad_x,
+                         colsum_out, mean_scratch)
+    dev = _check_some(grad_y=grad_y, grad_y_lower=grad_y_lower, grad_y_upper=grad_y_upper, grad_x=grad_x,
+                      colsum_out=colsum_out, mean_scratch=mean_scratch)
+    _run(_ms_bwd, dev, _po(grad_y), _po(grad_y_lower), _po(grad_y_upper), B, C, HW, 1 if training else 0, _po(grad_x),
+         _po(colsum_out), _po(mean_scratch))
 
 
 def _pair(v):

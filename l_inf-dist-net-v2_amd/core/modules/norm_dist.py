@@ -7,7 +7,7 @@ import math
 import torch
 import torch.nn as nn
 
-from core.norm_dist import norm_dist, bound_inf_dist, conv_norm_dist, conv_bound_inf_dist
+from core.norm_dist import norm_dist, bound_inf_dist, conv_norm_dist, conv_bound_inf_dist, mean_shift_bias
 from .basic_modules import MeanShift, apply_if_not_none
 
 
@@ -36,6 +36,14 @@ class NormDistBase(nn.Module):
         return self._shift_and_bias(x, lower, upper)
 
     def _shift_and_bias(self, x, lower, upper):
+        lead = next((t for t in (x, lower, upper) if t is not None), None)
+        if lead is not None and lead.is_cuda and lead.dtype == torch.float32 and \
+                (self.mean_shift is not None or self.bias is not None):
+            # one fused call for the mean shift (with its moving average) and both biases
+            ms = self.mean_shift
+            return mean_shift_bias(x, lower, upper, ms.running_mean if ms is not None else None,
+                                   ms.momentum if ms is not None else 0.0, ms.training if ms is not None else False,
+                                   ms.bias if ms is not None else None, self.bias)
         if self.mean_shift is not None:
             x, lower, upper = self.mean_shift(x, lower, upper)
         if self.bias is not None:

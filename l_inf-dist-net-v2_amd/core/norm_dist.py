@@ -247,6 +247,58 @@ def conv_bound_inf_dist(x_lower, x_upper, weight, kernel_size, dilation=1, paddi
                           unfold(x_upper, kernel_size, dilation, padding, stride), weight, groups, tag=tag)
 
 
+class MeanShiftBiasF(torch.autograd.Function):
+    """What follows the operator in every layer (reference: core/modules/norm_dist.py:35-38 and
+    core/modules/basic_modules.py:121-132), as one fused call: y* = t* - mean + bias1 + bias2 for t* in
+    (x, lower, upper), with mean the batch mean of x over (batch, position) in training (differentiable, also folded
+    into running_mean) or running_mean itself in evaluation; use_mean=False leaves the mean out (bias only).
+    Returns (y, y_lower, y_upper) with None where the input was None."""
+
+    @staticmethod
+    def forward(ctx, x, lower, upper, running_mean, momentum, training, use_mean, bias1, bias2):
+        batch_mean = bool(training and use_mean)
+        if batch_mean:
+            assert x is not None, 'Currently not supported'  # as the reference (core/modules/basic_modules.py:123)
+        x, lower, upper = (None if t is None else t.contiguous() for t in (x, lower, upper))
+        lead = next(t for t in (x, lower, upper) if t is not None)
+        C = lead.size(1)
+        ys = tuple(None if t is None else torch.empty_like(t) for t in (x, lower, upper))
+        mean_out = torch.empty(C, device=lead.device, dtype=torch.float32) if batch_mean else None
+        _C.mean_shift_forward(x, lower, upper, batch_mean, momentum, running_mean if use_mean else None,
+                              None if bias1 is None else bias1.detach(), None if bias2 is None else bias2.detach(),
+                              mean_out, *ys)
+        ctx.batch_mean = batch_mean
+        ctx.channels = C
+        ctx.bias_grad = (bias1 is not None and bias1.requires_grad, bias2 is not None and bias2.requires_grad)
+        ctx.set_materialize_grads(False)
+        return ys
+
+    @staticmethod
+    def backward(ctx, gy, gyl, gyu):
+        gy, gyl, gyu = (None if g is None else g.contiguous() for g in (gy, gyl, gyu))
+        lead = next((g for g in (gy, gyl, gyu) if g is not None), None)
+        if lead is None:
+            return (None,) * 9
+        want_cols = any(ctx.bias_grad)
+        new = lambda: torch.empty(ctx.channels, device=lead.device, dtype=torch.float32)
+        colsum = new() if want_cols else None
+        gx = gy
+        if ctx.batch_mean and ctx.needs_input_grad[0]:
+            if gy is None:
+                gy = torch.zeros_like(lead)  # only the bounds were used: grad_x is minus the mean of their gradients
+            gx = torch.empty_like(gy)
+            _C.mean_shift_backward(gy, gyl, gyu, True, gx, colsum, new())
+        elif want_cols:
+            _C.mean_shift_backward(gy, gyl, gyu, False, None, colsum, new())
+        return (gx, gyl, gyu, None, None, None, None,
+                colsum if ctx.bias_grad[0] else None, colsum if ctx.bias_grad[1] else None)
+
+
+def mean_shift_bias(x, lower, upper, running_mean, momentum, training, bias1=None, bias2=None):
+    """Fused mean shift (running_mean is not None) and bias add for CUDA tensors [B, C, HW]; see MeanShiftBiasF."""
+    return MeanShiftBiasF.apply(x, lower, upper, running_mean, momentum, training, running_mean is not None, bias1, bias2)
+
+
 def _grouped(t, groups):
     return t.view(t.size(0), groups, 1, -1, t.size(2))  # [B, G, 1, CI/G, HW]
 

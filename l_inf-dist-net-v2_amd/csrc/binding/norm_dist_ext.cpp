@@ -328,6 +328,48 @@ void conv_bound_inf_dist_backward_input_weight(const Tensor& grad_outputL, const
              "conv_bound_inf_dist_backward_input_weight");
 }
 
+// ---- mean shift and bias (no kernel of its own in the reference: core/modules/basic_modules.py:121-132) ------------
+// absent tensors are passed as None
+using OptTensor = c10::optional<Tensor>;
+const float* FO(const OptTensor& t) { return t.has_value() ? t->data_ptr<float>() : nullptr; }
+float* FMO(OptTensor& t) { return t.has_value() ? t->data_ptr<float>() : nullptr; }
+
+int check_optional(std::initializer_list<std::pair<const char*, const OptTensor*>> args) {
+    int dev = -1;
+    for (const auto& a : args) {
+        if (!a.second->has_value()) continue;
+        const Tensor& t = **a.second;
+        TORCH_CHECK(t.is_cuda(), a.first, " must be a CUDA tensor");
+        TORCH_CHECK(t.is_contiguous(), a.first, " must be contiguous");
+        TORCH_CHECK(t.scalar_type() == torch::kFloat32, a.first, " must have dtype torch.float32");
+        if (dev < 0) dev = t.get_device();
+        TORCH_CHECK(t.get_device() == dev, a.first, " is on device ", t.get_device(), ", expected ", dev);
+    }
+    TORCH_CHECK(dev >= 0, "at least one tensor is required");
+    return dev;
+}
+
+void mean_shift_forward(const OptTensor& x, const OptTensor& lower, const OptTensor& upper, int B, int C, int HW,
+                        bool training, double momentum, OptTensor running_mean, const OptTensor& bias1,
+                        const OptTensor& bias2, OptTensor mean_out, OptTensor y, OptTensor y_lower, OptTensor y_upper) {
+    const int dev = check_optional({{"x", &x}, {"lower", &lower}, {"upper", &upper}, {"running_mean", &running_mean},
+                                    {"bias1", &bias1}, {"bias2", &bias2}, {"mean_out", &mean_out}, {"y", &y},
+                                    {"y_lower", &y_lower}, {"y_upper", &y_upper}});
+    Launch L(dev);
+    raise_on(ndist_mean_shift_forward(FO(x), FO(lower), FO(upper), B, C, HW, training ? 1 : 0, (float)momentum,
+                                      FMO(running_mean), FO(bias1), FO(bias2), FMO(mean_out), FMO(y), FMO(y_lower),
+                                      FMO(y_upper), L.stream), "mean_shift_forward");
+}
+
+void mean_shift_backward(const OptTensor& grad_y, const OptTensor& grad_y_lower, const OptTensor& grad_y_upper, int B,
+                         int C, int HW, bool training, OptTensor grad_x, OptTensor colsum_out, OptTensor mean_scratch) {
+    const int dev = check_optional({{"grad_y", &grad_y}, {"grad_y_lower", &grad_y_lower}, {"grad_y_upper", &grad_y_upper},
+                                    {"grad_x", &grad_x}, {"colsum_out", &colsum_out}, {"mean_scratch", &mean_scratch}});
+    Launch L(dev);
+    raise_on(ndist_mean_shift_backward(FO(grad_y), FO(grad_y_lower), FO(grad_y_upper), B, C, HW, training ? 1 : 0,
+                                       FMO(grad_x), FMO(colsum_out), FMO(mean_scratch), L.stream), "mean_shift_backward");
+}
+
 // ---- process-wide switches and aids ------------------------------------------------------------------------------
 double last_kernel_ms() {
     float ms = 0.f;
@@ -370,6 +412,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("conv_inf_dist_backward_input_weight", &conv_inf_dist_backward_input_weight);
     m.def("conv_bound_inf_dist_backward_input", &conv_bound_inf_dist_backward_input);
     m.def("conv_bound_inf_dist_backward_input_weight", &conv_bound_inf_dist_backward_input_weight);
+    m.def("mean_shift_forward", &mean_shift_forward);
+    m.def("mean_shift_backward", &mean_shift_backward);
     m.def("version", []() { return ndist_version(); });
     m.def("set_profiling", [](bool on) { ndist_set_profiling(on ? 1 : 0); });
     m.def("last_kernel_ms", &last_kernel_ms);
