@@ -165,6 +165,18 @@ int ndist_bound_inf_dist_backward_input_weight(const float* grad_outputL, const 
                                                float* grad_inputL, float* grad_inputU, float* grad_weight,
                                                ndist_stream_t stream);
 
+/* ---- a layer's distance and its interval bounds in one call ---------------------------------------------------
+ * No counterpart in the reference's kernel interface: its layers call inf_dist::forward[_nograd] and
+ * bound_inf_dist::forward[_nograd] one after the other on the same weights (core/modules/norm_dist.py:30-34), which is
+ * what certification does on every layer.  These entry points compute exactly what those two calls compute (same
+ * values, same codes) and share the pre-pass over the weights between them where the k-tile skipping variants run. */
+int ndist_inf_and_bound_forward_nograd(const float* input, const float* inputL, const float* inputU, const float* weight,
+                                       int B, int CO, int CI, int G, int HW, float* output, float* outputL,
+                                       float* outputU, ndist_stream_t stream);
+int ndist_inf_and_bound_forward(const float* input, const float* inputL, const float* inputU, const float* weight, int B,
+                                int CO, int CI, int G, int HW, float* output, int32_t* pos, float* outputL,
+                                float* outputU, int32_t* posL, int32_t* posU, ndist_stream_t stream);
+
 /* ---- mean shift and bias of a distance layer ------------------------------------------------------------------
  * The reference has no kernel of its own here: every layer follows the operator with MeanShift and a bias add
  * written in torch primitives (core/modules/norm_dist.py:35-38, core/modules/basic_modules.py:121-132).  These two

@@ -81,6 +81,8 @@ _bnd_fwd_ng = _sig("ndist_bound_inf_dist_forward_nograd", _P, _P, _P, *_DIMS, _P
 _bnd_fwd = _sig("ndist_bound_inf_dist_forward", _P, _P, _P, *_DIMS, _P, _P, _P, _P, _P)
 _bnd_bwd_x = _sig("ndist_bound_inf_dist_backward_input", _P, _P, _P, _P, *_DIMS, _P, _P, _P)
 _bnd_bwd_xw = _sig("ndist_bound_inf_dist_backward_input_weight", _P, _P, _P, _P, *_DIMS, _P, _P, _P, _P)
+_joint_ng = _sig("ndist_inf_and_bound_forward_nograd", _P, _P, _P, _P, *_DIMS, _P, _P, _P, _P)
+_joint = _sig("ndist_inf_and_bound_forward", _P, _P, _P, _P, *_DIMS, _P, _P, _P, _P, _P, _P, _P)
 _ms_fwd = _sig("ndist_mean_shift_forward", _P, _P, _P, _I, _I, _I, _I, _F, _P, _P, _P, _P, _P, _P, _P, _P)
 _ms_bwd = _sig("ndist_mean_shift_backward", _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P)
 _unfold_fwd = _sig("ndist_unfold_forward", _P, *([_I] * 12), _P, _P)
@@ -320,6 +322,31 @@ def bound_inf_dist_backward_input_weight(grad_outputL, grad_outputU, posL, posU,
     B, CO, CI, HW = grad_outputL.size(0), grad_outputL.size(1), grad_weight.size(1) * G, grad_outputL.size(2)
     _run(_bnd_bwd_xw, dev, _p(grad_outputL), _p(grad_outputU), _p(posL), _p(posU), B, CO, CI, G, HW,
          _p(grad_inputL), _p(grad_inputU), _p(grad_weight))
+
+
+def inf_and_bound_forward_nograd(input, inputL, inputU, weight, output, outputL, outputU, G):
+    """inf_dist_forward_nograd(input) and bound_inf_dist_forward_nograd(inputL, inputU) against the same weights in one
+    call: the two calls a layer makes under certification (reference: core/modules/norm_dist.py:30-34), with the
+    pre-pass over the weights shared."""
+    if _ext is not None:
+        return _ext_call(_ext.inf_and_bound_forward_nograd, input, inputL, inputU, weight, output, outputL, outputU, G)
+    dev = _check({}, input=input, inputL=inputL, inputU=inputU, weight=weight, output=output, outputL=outputL,
+                 outputU=outputU)
+    B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
+    _run(_joint_ng, dev, _p(input), _p(inputL), _p(inputU), _p(weight), B, CO, CI, G, HW, _p(output), _p(outputL),
+         _p(outputU))
+
+
+def inf_and_bound_forward(input, inputL, inputU, weight, output, pos, outputL, outputU, posL, posU, G):
+    """The same with the arg-max codes of all three reductions (inf_dist_forward + bound_inf_dist_forward)."""
+    if _ext is not None:
+        return _ext_call(_ext.inf_and_bound_forward, input, inputL, inputU, weight, output, pos, outputL, outputU, posL,
+                         posU, G)
+    dev = _check(_INT, input=input, inputL=inputL, inputU=inputU, weight=weight, output=output, pos=pos,
+                 outputL=outputL, outputU=outputU, posL=posL, posU=posU)
+    B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
+    _run(_joint, dev, _p(input), _p(inputL), _p(inputU), _p(weight), B, CO, CI, G, HW, _p(output), _p(pos), _p(outputL),
+         _p(outputU), _p(posL), _p(posU))
 
 
 def _po(t):

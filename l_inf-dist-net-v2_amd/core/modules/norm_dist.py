@@ -7,7 +7,8 @@ import math
 import torch
 import torch.nn as nn
 
-from core.norm_dist import norm_dist, bound_inf_dist, conv_norm_dist, conv_bound_inf_dist, mean_shift_bias
+from core.norm_dist import (norm_dist, bound_inf_dist, conv_norm_dist, conv_bound_inf_dist, mean_shift_bias,
+                            inf_dist_with_bounds)
 from .basic_modules import MeanShift, apply_if_not_none
 
 
@@ -28,6 +29,10 @@ class NormDistBase(nn.Module):
         self.tag = NormDistBase.tag
 
     def forward(self, x=None, lower=None, upper=None):
+        if x is not None and lower is not None and upper is not None and math.isinf(self.p) and x.is_cuda:
+            # the distance and its bounds against the same weights: one call (shares the pre-pass over the weights)
+            x, lower, upper = inf_dist_with_bounds(x, lower, upper, self.weight, self.groups, tag=self.tag)
+            return self._shift_and_bias(x, lower, upper)
         if x is not None:
             x = norm_dist(x, self.weight, self.p, self.groups, tag=self.tag)
         if lower is not None and upper is not None:

@@ -247,6 +247,24 @@ def conv_bound_inf_dist(x_lower, x_upper, weight, kernel_size, dilation=1, paddi
                           unfold(x_upper, kernel_size, dilation, padding, stride), weight, groups, tag=tag)
 
 
+def inf_dist_with_bounds(x, x_lower, x_upper, weight, groups=1, tag=None):
+    """(y, y_lower, y_upper): the infinity distance of x and the interval bounds of the box (x_lower, x_upper) against
+    the same weights: what a layer computes under certification (reference: core/modules/norm_dist.py:30-34, two
+    operator calls).  Without gradients the two run as one library call that shares the pre-pass over the weights;
+    with gradients they are the two autograd operators."""
+    tensors = (x, x_lower, x_upper, weight)
+    if (all(t.is_cuda and t.dtype == torch.float32 for t in tensors)
+            and not (torch.is_grad_enabled() and any(t.requires_grad for t in tensors))):
+        x, x_lower, x_upper, weight = (t.contiguous() for t in tensors)
+        y = _new_output(x, weight)
+        y_lower, y_upper = torch.empty_like(y), torch.empty_like(y)
+        _C.inf_and_bound_forward_nograd(x, x_lower, x_upper, weight, y, y_lower, y_upper, groups)
+        return y, y_lower, y_upper
+    y = norm_dist(x, weight, INF, groups, tag=tag)
+    y_lower, y_upper = bound_inf_dist(x_lower, x_upper, weight, groups, tag=tag)
+    return y, y_lower, y_upper
+
+
 class MeanShiftBiasF(torch.autograd.Function):
     """What follows the operator in every layer (reference: core/modules/norm_dist.py:35-38 and
     core/modules/basic_modules.py:121-132), as one fused call: y* = t* - mean + bias1 + bias2 for t* in

@@ -211,6 +211,36 @@ void bound_inf_dist_backward_input_weight(const Tensor& grad_outputL, const Tens
              "bound_inf_dist_backward_input_weight");
 }
 
+// a layer's distance and its interval bounds in one call (pre-pass over the weights shared); no counterpart in the
+// reference's extension, whose layers make the two calls one after the other (core/modules/norm_dist.py:30-34)
+void inf_and_bound_forward_nograd(const Tensor& input, const Tensor& inputL, const Tensor& inputU, const Tensor& weight,
+                                  Tensor& output, Tensor& outputL, Tensor& outputU, int G) {
+    const int dev = check_all({{"input", input, false}, {"inputL", inputL, false}, {"inputU", inputU, false},
+                               {"weight", weight, false}, {"output", output, false}, {"outputL", outputL, false},
+                               {"outputU", outputU, false}});
+    need3d(input, "input"); need3d(output, "output");
+    TORCH_CHECK(input.sizes() == inputL.sizes() && input.sizes() == inputU.sizes(), "input and its bounds must have the same shape");
+    TORCH_CHECK(output.sizes() == outputL.sizes() && output.sizes() == outputU.sizes(), "the three outputs must have the same shape");
+    Launch L(dev);
+    raise_on(ndist_inf_and_bound_forward_nograd(F(input), F(inputL), F(inputU), F(weight), input.size(0), output.size(1),
+                                                input.size(1), G, input.size(2), FM(output), FM(outputL), FM(outputU),
+                                                L.stream), "inf_and_bound_forward_nograd");
+}
+
+void inf_and_bound_forward(const Tensor& input, const Tensor& inputL, const Tensor& inputU, const Tensor& weight,
+                           Tensor& output, Tensor& pos, Tensor& outputL, Tensor& outputU, Tensor& posL, Tensor& posU, int G) {
+    const int dev = check_all({{"input", input, false}, {"inputL", inputL, false}, {"inputU", inputU, false},
+                               {"weight", weight, false}, {"output", output, false}, {"pos", pos, true},
+                               {"outputL", outputL, false}, {"outputU", outputU, false}, {"posL", posL, true},
+                               {"posU", posU, true}});
+    need3d(input, "input"); need3d(output, "output");
+    TORCH_CHECK(input.sizes() == inputL.sizes() && input.sizes() == inputU.sizes(), "input and its bounds must have the same shape");
+    Launch L(dev);
+    raise_on(ndist_inf_and_bound_forward(F(input), F(inputL), F(inputU), F(weight), input.size(0), output.size(1),
+                                         input.size(1), G, input.size(2), FM(output), IM(pos), FM(outputL), FM(outputU),
+                                         IM(posL), IM(posU), L.stream), "inf_and_bound_forward");
+}
+
 // ---- patch extraction and the convolutional layer without the unfolded tensor ------------------------------------
 // geometry: (kernel_h, kernel_w, dilation_h, dilation_w, padding_h, padding_w, stride_h, stride_w)
 using Geo = std::vector<int64_t>;
@@ -412,6 +442,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("conv_inf_dist_backward_input_weight", &conv_inf_dist_backward_input_weight);
     m.def("conv_bound_inf_dist_backward_input", &conv_bound_inf_dist_backward_input);
     m.def("conv_bound_inf_dist_backward_input_weight", &conv_bound_inf_dist_backward_input_weight);
+    m.def("inf_and_bound_forward_nograd", &inf_and_bound_forward_nograd);
+    m.def("inf_and_bound_forward", &inf_and_bound_forward);
     m.def("mean_shift_forward", &mean_shift_forward);
     m.def("mean_shift_backward", &mean_shift_backward);
     m.def("version", []() { return ndist_version(); });

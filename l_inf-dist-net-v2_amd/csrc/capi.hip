@@ -298,6 +298,29 @@ int ndist_bound_inf_dist_backward_input_weight(const float* grad_outputL, const 
                                  (hipStream_t)stream);
 }
 
+int ndist_inf_and_bound_forward_nograd(const float* input, const float* inputL, const float* inputU, const float* weight,
+                                       int B, int CO, int CI, int G, int HW, float* output, float* outputL,
+                                       float* outputU, ndist_stream_t stream) {
+    NDIST_REQUIRE(input); NDIST_REQUIRE(inputL); NDIST_REQUIRE(inputU); NDIST_REQUIRE(weight);
+    NDIST_REQUIRE(output); NDIST_REQUIRE(outputL); NDIST_REQUIRE(outputU);
+    Geom s;
+    if (int rc = make_geom(B, CO, CI, G, HW, &s)) return rc;
+    return launch_inf_bound_forward(input, inputL, inputU, weight, s, output, nullptr, outputL, outputU, nullptr, nullptr,
+                                    (hipStream_t)stream);
+}
+
+int ndist_inf_and_bound_forward(const float* input, const float* inputL, const float* inputU, const float* weight, int B,
+                                int CO, int CI, int G, int HW, float* output, int32_t* pos, float* outputL,
+                                float* outputU, int32_t* posL, int32_t* posU, ndist_stream_t stream) {
+    NDIST_REQUIRE(input); NDIST_REQUIRE(inputL); NDIST_REQUIRE(inputU); NDIST_REQUIRE(weight);
+    NDIST_REQUIRE(output); NDIST_REQUIRE(outputL); NDIST_REQUIRE(outputU);
+    NDIST_REQUIRE(pos); NDIST_REQUIRE(posL); NDIST_REQUIRE(posU);
+    Geom s;
+    if (int rc = make_geom(B, CO, CI, G, HW, &s)) return rc;
+    return launch_inf_bound_forward(input, inputL, inputU, weight, s, output, pos, outputL, outputU, posL, posU,
+                                    (hipStream_t)stream);
+}
+
 int ndist_unfold_forward(const float* input, int B, int C, int H, int W, int kernel_h, int kernel_w, int dilation_h,
                          int dilation_w, int padding_h, int padding_w, int stride_h, int stride_w, float* output,
                          ndist_stream_t stream) {

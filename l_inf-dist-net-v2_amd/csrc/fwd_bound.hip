@@ -164,7 +164,7 @@ __global__ __launch_bounds__(256) void bound_rescan_kernel(const float* __restri
 }
 
 int launch_bound_forward(const float* xl, const float* xu, const float* w, const Geom& s, float* yl, float* yu,
-                         int32_t* pl, int32_t* pu, hipStream_t st, const UnfoldGeom* cv) {
+                         int32_t* pl, int32_t* pu, hipStream_t st, const UnfoldGeom* cv, const WeightSeeds* wpre) {
     FwdParams P{};
     PatchMap pm{};
     if (cv != nullptr) {
@@ -181,9 +181,7 @@ int launch_bound_forward(const float* xl, const float* xu, const float* w, const
     P.pos2 = pu;
     P.s = s;
     // large fully-connected problems: seeds and k-tile bounds, as in launch_inf_forward
-    const double pairs = (double)s.M * s.COg * s.G * s.CIg;
-    const bool bounded = cv == nullptr && s.HW == 1 && !skinny_applies(s) && skip_override_limit(1) > 0 &&
-                         ((pairs >= 2e8 && s.M >= kMinSeededRows) || skip_forced_on());
+    const bool bounded = cv == nullptr && seeded_forward_applies(s);
     if (!bounded && pl == nullptr) return launch_fwd_conv<OpBound<false>, CfgBoundN, CfgMid, CfgSmall>(P, st);
     KernelTimer timer(st);  // pre-passes + tiled kernel + rescan
     float* scratch = nullptr;
@@ -191,7 +189,7 @@ int launch_bound_forward(const float* xl, const float* xu, const float* w, const
         const size_t total = (size_t)s.M * s.COg * s.G;
         NDIST_HIP_TRY(scratch_alloc((void**)&scratch, (seed_scratch_floats(s) + total) * sizeof(float), st));
         SeedBuffers sb{};
-        const int rs = launch_seeds(xl, w, s, scratch, nullptr, 0, st, &sb, xu);
+        const int rs = launch_seeds(xl, w, s, scratch, nullptr, 0, st, &sb, xu, wpre);
         if (rs) {
             (void)scratch_free(scratch, st);
             return rs;
@@ -229,6 +227,25 @@ int launch_bound_forward(const float* xl, const float* xu, const float* w, const
     else return 2;
 #undef NDIST_BOUND_RESCAN
     return hip_failed(hipGetLastError()) ? 4 : 0;
+}
+
+// A layer's distance and its interval bounds in one call (certification runs both on every layer with the same
+// weights, reference: core/modules/norm_dist.py:30-34): on problems large enough for the k-tile skipping variants the
+// pre-pass over w (the largest of the pre-passes: it reads all of w) runs once and serves both operators.
+int launch_inf_bound_forward(const float* x, const float* xl, const float* xu, const float* w, const Geom& s, float* out,
+                             int32_t* pos, float* yl, float* yu, int32_t* pl, int32_t* pu, hipStream_t st) {
+    if (!seeded_forward_applies(s)) {
+        const int rc = launch_inf_forward(x, w, s, out, pos, st);
+        return rc ? rc : launch_bound_forward(xl, xu, w, s, yl, yu, pl, pu, st);
+    }
+    float* block = nullptr;
+    NDIST_HIP_TRY(scratch_alloc((void**)&block, weight_seed_floats(s) * sizeof(float), st));
+    WeightSeeds ws{};
+    int rc = launch_weight_seeds(w, s, block, nullptr, 0, st, &ws);
+    if (!rc) rc = launch_inf_forward(x, w, s, out, pos, st, nullptr, &ws);
+    if (!rc) rc = launch_bound_forward(xl, xu, w, s, yl, yu, pl, pu, st, nullptr, &ws);
+    if (hip_failed(scratch_free(block, st)) && !rc) rc = 4;
+    return rc;
 }
 
 }  // namespace ndist

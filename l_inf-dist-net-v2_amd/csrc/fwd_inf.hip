@@ -140,8 +140,14 @@ __global__ __launch_bounds__(256) void inf_rescan_kernel(const float* __restrict
     pos[o] = (int32_t)code;
 }
 
+bool seeded_forward_applies(const Geom& s) {
+    const double pairs = (double)s.M * s.COg * s.G * s.CIg;
+    return s.HW == 1 && !skinny_applies(s) && skip_override_limit(1) > 0 &&
+           ((pairs >= 2e8 && s.M >= kMinSeededRows) || skip_forced_on());
+}
+
 int launch_inf_forward(const float* x, const float* w, const Geom& s, float* out, int32_t* pos, hipStream_t st,
-                       const UnfoldGeom* cv) {
+                       const UnfoldGeom* cv, const WeightSeeds* wpre) {
     FwdParams P{};
     P.x = x;
     P.w = w;
@@ -158,15 +164,13 @@ int launch_inf_forward(const float* x, const float* w, const Geom& s, float* out
     // that skips the k-tiles which cannot matter (most of them, unless the largest |x - w| are far below
     // max|x| + max|w| everywhere).  NORM_DIST_SKIP=0 / ndist_set_skip_mode(0, ..) switches this off, 1 forces it on
     // for small problems too.
-    const double pairs = (double)s.M * s.COg * s.G * s.CIg;
-    const bool bounded = cv == nullptr && s.HW == 1 && !skinny_applies(s) && skip_override_limit(1) > 0 &&
-                         ((pairs >= 2e8 && s.M >= kMinSeededRows) || skip_forced_on());
+    const bool bounded = cv == nullptr && seeded_forward_applies(s);
     float* scratch = nullptr;
     KernelTimer timer(st);  // pre-passes + tiled kernel + rescan
     if (bounded) {
         NDIST_HIP_TRY(scratch_alloc((void**)&scratch, seed_scratch_floats(s) * sizeof(float), st));
         SeedBuffers sb{};
-        const int rs = launch_seeds(x, w, s, scratch, nullptr, 0, st, &sb);
+        const int rs = launch_seeds(x, w, s, scratch, nullptr, 0, st, &sb, nullptr, wpre);
         if (rs) {
             (void)scratch_free(scratch, st);
             return rs;

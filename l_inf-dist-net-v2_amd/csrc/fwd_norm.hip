@@ -612,8 +612,31 @@ size_t seed_scratch_floats(const Geom& s) {
     return (2 + (size_t)ceil_div(s.CIg, 32)) * (rows + wrows) + total;
 }
 
+size_t weight_seed_floats(const Geom& s) {
+    return (2 + (size_t)ceil_div(s.CIg, 32)) * ((size_t)s.COg * s.G);
+}
+
+int launch_weight_seeds(const float* w, const Geom& s, float* base, const int* gate, int gate_limit, hipStream_t st,
+                        WeightSeeds* out) {
+    const long wrows = (long)s.COg * s.G;
+    const int ntile = ceil_div(s.CIg, 32);
+    out->seed_w = base;
+    out->seed_wk = reinterpret_cast<int32_t*>(base + wrows);
+    out->tile_w = reinterpret_cast<float*>(out->seed_wk + wrows);
+    // the rows of w: the row kernel on the geometry of a [CO, CIg] matrix
+    Geom ws{};
+    ws.B = ws.M = (int)wrows;
+    ws.HW = 1;
+    ws.G = 1;
+    ws.CIg = s.CIg;
+    ws.COg = 1;
+    hipLaunchKernelGGL(norm_seed_kernel, dim3((unsigned)((wrows + 3) / 4)), dim3(256), 0, st, w, (const float*)nullptr, ws,
+                       out->seed_w, out->seed_wk, out->tile_w, ntile, gate, gate_limit);
+    return hip_failed(hipGetLastError()) ? 4 : 0;
+}
+
 int launch_seeds(const float* x, const float* w, const Geom& s, float* base, const int* gate, int gate_limit,
-                 hipStream_t st, SeedBuffers* out, const float* x2) {
+                 hipStream_t st, SeedBuffers* out, const float* x2, const WeightSeeds* wpre) {
     const long rows = (long)s.M * s.G, wrows = (long)s.COg * s.G, total = (long)s.M * s.COg * s.G;
     const int ntile = ceil_div(s.CIg, 32);
     int rc = 0;
@@ -624,26 +647,33 @@ int launch_seeds(const float* x, const float* w, const Geom& s, float* base, con
     float* seed = reinterpret_cast<float*>(seed_wk + wrows);
     float* tile_x = seed + total;
     float* tile_w = tile_x + rows * ntile;
+    float* const after_tiles = tile_w + wrows * ntile;
     hipLaunchKernelGGL(norm_seed_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, x, x2, s, seed_x, seed_k,
                        tile_x, ntile, gate, gate_limit);
     if (hip_failed(hipGetLastError())) rc = 4;
-    // the rows of w: the same kernel on the geometry of a [CO, CIg] matrix
-    Geom ws{};
-    ws.B = ws.M = (int)wrows;
-    ws.HW = 1;
-    ws.G = 1;
-    ws.CIg = s.CIg;
-    ws.COg = 1;
-    hipLaunchKernelGGL(norm_seed_kernel, dim3((unsigned)((wrows + 3) / 4)), dim3(256), 0, st, w, (const float*)nullptr, ws,
-                       seed_w, seed_wk, tile_w, ntile, gate, gate_limit);
-    if (hip_failed(hipGetLastError())) rc = 4;
+    if (wpre != nullptr) {
+        seed_w = wpre->seed_w;
+        seed_wk = wpre->seed_wk;
+        tile_w = wpre->tile_w;
+    } else {
+        // the rows of w: the same kernel on the geometry of a [CO, CIg] matrix
+        Geom ws{};
+        ws.B = ws.M = (int)wrows;
+        ws.HW = 1;
+        ws.G = 1;
+        ws.CIg = s.CIg;
+        ws.COg = 1;
+        hipLaunchKernelGGL(norm_seed_kernel, dim3((unsigned)((wrows + 3) / 4)), dim3(256), 0, st, w, (const float*)nullptr,
+                           ws, seed_w, seed_wk, tile_w, ntile, gate, gate_limit);
+        if (hip_failed(hipGetLastError())) rc = 4;
+    }
     const int nmb = ceil_div(s.M, 64), nnb = ceil_div(s.COg, 64);
     float* seed2 = nullptr;
     if (x2 == nullptr) {
         hipLaunchKernelGGL(norm_seed_outputs_kernel, dim3((unsigned)((long)nmb * nnb * s.G)), dim3(256), 0, st, x, w, s,
                            seed_x, seed_k, seed_w, seed_wk, seed, nmb, nnb, gate, gate_limit);
     } else {  // interval bounds (ungated): the second seed array lies behind the tile bounds
-        seed2 = tile_w + wrows * ntile;
+        seed2 = after_tiles;
         hipLaunchKernelGGL(bound_seed_outputs_kernel, dim3((unsigned)((long)nmb * nnb * s.G)), dim3(256), 0, st, x, x2, w,
                            s, seed_k, seed_w, seed_wk, seed, seed2, nmb, nnb);
     }

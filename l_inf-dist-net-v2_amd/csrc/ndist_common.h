@@ -115,9 +115,20 @@ struct SeedBuffers {
     float* tile_w;
     int ntile;
 };
+// The part of the pre-passes that depends on w alone (per row of w: largest element, its k, tile maxima): two
+// operators called on the same weights (a layer's distance and its interval bounds) can share it.
+struct WeightSeeds {
+    float* seed_w;
+    int32_t* seed_wk;
+    float* tile_w;
+};
 size_t seed_scratch_floats(const Geom& s);
+size_t weight_seed_floats(const Geom& s);
+int launch_weight_seeds(const float* w, const Geom& s, float* base, const int* gate, int gate_limit, hipStream_t st,
+                        WeightSeeds* out);
+// `wpre`: weight rows already done by launch_weight_seeds (their part of `base` then stays unused)
 int launch_seeds(const float* x, const float* w, const Geom& s, float* base, const int* gate, int gate_limit,
-                 hipStream_t st, SeedBuffers* out, const float* x2 = nullptr);
+                 hipStream_t st, SeedBuffers* out, const float* x2 = nullptr, const WeightSeeds* wpre = nullptr);
 
 #define NDIST_HIP_TRY(expr)                                        \
     do {                                                           \
@@ -210,10 +221,15 @@ int launch_fold(const float* gout, const UnfoldGeom& u, float* gx, hipStream_t s
 // The forward launchers take an optional patch geometry `cv`: x (xl, xu) are then images [B, C, H, W], s describes
 // the unfolded problem (CIg = C / G * kh * kw, HW = OH * OW) and the kernels extract the patches while loading.
 int launch_inf_forward(const float* x, const float* w, const Geom& s, float* out, int32_t* pos, hipStream_t st,
-                       const UnfoldGeom* cv = nullptr);
+                       const UnfoldGeom* cv = nullptr, const WeightSeeds* wpre = nullptr);
 int launch_bound_forward(const float* xl, const float* xu, const float* w, const Geom& s,
                          float* yl, float* yu, int32_t* pl, int32_t* pu, hipStream_t st,
-                         const UnfoldGeom* cv = nullptr);
+                         const UnfoldGeom* cv = nullptr, const WeightSeeds* wpre = nullptr);
+// true when the two launchers above would run their seeded (k-tile skipping) variants on this problem
+bool seeded_forward_applies(const Geom& s);
+// the distance of x and the interval bounds of (xl, xu) against the same weights, pre-passes over w shared
+int launch_inf_bound_forward(const float* x, const float* xl, const float* xu, const float* w, const Geom& s, float* out,
+                             int32_t* pos, float* yl, float* yu, int32_t* pl, int32_t* pu, hipStream_t st);
 int launch_norm_forward(const float* x, const float* w, const float* max_in, const Geom& s, float* out, float p,
                         hipStream_t st);
 int launch_norm_backward(const float* gout, const float* x, const float* w, const float* out, const Geom& s,
