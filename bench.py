@@ -226,9 +226,12 @@ def other_workloads(torch, _C, xd, wd, gd):
 
 
 def run_part(torch, _C, args, xd, wd, gd):
-    """One entry point, called --steps times through the binding on pre-allocated outputs (for rocprofv3 runs)."""
-    out = torch.empty(B, CO, 1, device=xd.device)
-    pos = torch.empty(B, CO, 1, device=xd.device, dtype=torch.int32)
+    """One entry point, called --steps times through the binding on pre-allocated outputs (for rocprofv3 runs);
+    --batch takes the first rows of the benchmark's batch (64: the small-batch cases)."""
+    nb = args.batch
+    xd, gd = xd[:nb].contiguous(), gd[:nb].contiguous()
+    out = torch.empty(nb, CO, 1, device=xd.device)
+    pos = torch.empty(nb, CO, 1, device=xd.device, dtype=torch.int32)
     gx = torch.empty_like(xd)
     gw = torch.empty_like(wd)
     _C.norm_dist_forward(xd, wd, out, 1, 8.0)
@@ -238,6 +241,7 @@ def run_part(torch, _C, args, xd, wd, gd):
         "p8_fwd": lambda: _C.norm_dist_forward(xd, wd, out, 1, 8.0),
         "p8_bwd": lambda: _C.norm_dist_backward_input_weight(gd, xd, wd, out8, gx, gw, 1, 8.0),
         "inf_fwd": lambda: _C.inf_dist_forward(xd, wd, out, pos, 1),
+        "inf_fwd_nograd": lambda: _C.inf_dist_forward_nograd(xd, wd, out, 1),
         "inf_bwd": lambda: _C.inf_dist_backward_input_weight(gd, pos, gx, gw, 1),
     }
     if args.part == "copy":
@@ -254,7 +258,8 @@ def run_part(torch, _C, args, xd, wd, gd):
         fn()
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    print(json.dumps({"part": args.part, "ms_per_call": round(ms, 4), "steps": args.steps, "warmup": args.warmup}))
+    print(json.dumps({"part": args.part, "batch": nb, "ms_per_call": round(ms, 4), "steps": args.steps,
+                      "warmup": args.warmup}))
 
 
 def main():
@@ -264,8 +269,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--cpu-cols", type=int, default=1024, help="output features of the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-other", action="store_true", help="skip the secondary workloads (general p, IBP, MLP, conv)")
-    ap.add_argument("--part", default="all", choices=["all", "p8_fwd", "p8_bwd", "inf_fwd", "inf_bwd", "copy", "other"],
+    ap.add_argument("--part", default="all",
+                    choices=["all", "p8_fwd", "p8_bwd", "inf_fwd", "inf_fwd_nograd", "inf_bwd", "copy", "other"],
                     help="profiling aid: run only one entry point of the step, --steps times, on pre-allocated outputs")
+    ap.add_argument("--batch", type=int, default=B, help="with --part: rows of the batch to use (e.g. 64)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus %d is not supported (no collective is built or used)"
