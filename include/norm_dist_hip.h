@@ -68,6 +68,13 @@ int ndist_last_kernel_ms(float* ms);
  * the environment: NORM_DIST_SKIP, NORM_DIST_BWD_BOUNDS = 0 / 1.  Results agree within the operator's tolerance
  * whichever variant runs. */
 void ndist_set_skip_mode(int skip, int bounds);
+/* Tuning and test aid, no counterpart in the reference.  On the problems whose p = inf forward skips k-tiles the
+ * library first finds out on the device whether a few 32-wide k-tiles per row of x, or per row of w, decide every
+ * maximum (activations with a few outliers against small weights; weights with one large planted entry per row) and
+ * then computes the outputs from those tiles alone; results are bit-identical either way.  mode: -1 the counts
+ * decide (default), 0 never, 1 always the cheaper side, 2 always the rows of x, 3 always the rows of w.
+ * Process-wide; initial value from NORM_DIST_HOT. */
+void ndist_set_hot_mode(int mode);
 /* No counterpart in the reference (PyTorch's caching allocator plays this role there).  Entry points that need
  * temporary device memory (finite-p backward, forwards whose k range is split over workgroups, the large-p paths,
  * the conv fallback) take it from arenas the library keeps per (device, stream): allocated with hipMalloc the first

@@ -58,6 +58,8 @@ _lib.ndist_set_profiling.argtypes = [ctypes.c_int]
 _lib.ndist_set_profiling.restype = None
 _lib.ndist_set_skip_mode.argtypes = [ctypes.c_int, ctypes.c_int]
 _lib.ndist_set_skip_mode.restype = None
+_lib.ndist_set_hot_mode.argtypes = [ctypes.c_int]
+_lib.ndist_set_hot_mode.restype = None
 _lib.ndist_release_scratch.argtypes = []
 _lib.ndist_release_scratch.restype = ctypes.c_int
 _lib.ndist_last_kernel_ms.argtypes = [ctypes.POINTER(ctypes.c_float)]
@@ -135,6 +137,12 @@ def set_skip_mode(skip=-1, bounds=-1):
     """Tuning / test aid: -1 lets the device-side probes choose the large-p kernel variants (default), 0 / 1 forces
     the pair-skipping variants off / on; `bounds` likewise for the two skipping variants of the backward."""
     _lib.ndist_set_skip_mode(int(skip), int(bounds))
+
+
+def set_hot_mode(mode=-1):
+    """Tuning / test aid for the p = inf forward through hot k-tiles: -1 the device-side counts decide (default),
+    0 never, 1 always the cheaper side, 2 always by the rows of x, 3 always by the rows of w."""
+    _lib.ndist_set_hot_mode(int(mode))
 
 
 def release_scratch():

@@ -148,6 +148,7 @@ int ndist_last_hip_error(void) { return g_last_hip_error; }
 void ndist_set_profiling(int enable) { g_profiling.store(enable ? 1 : 0); }
 
 void ndist_set_skip_mode(int skip, int bounds) { set_skip_mode(skip, bounds); }
+void ndist_set_hot_mode(int mode) { set_hot_mode(mode); }
 
 int ndist_release_scratch(void) { return scratch_release_all(); }
 

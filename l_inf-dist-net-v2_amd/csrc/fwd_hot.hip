@@ -1,0 +1,363 @@
+// Forward of the infinity distance through "hot" k-tiles only (fully-connected layout, HW == 1).
+// Serves inf_dist::forward / forward_nograd of the reference (core/cuda/inf_dist_cuda.cu:14-198,248-317) on data
+// whose largest |x - w| are decided by few k: results are bit-identical to the dense kernels (values and codes).
+//
+// out[m, n] = max_k |x[m, k] - w[n, k]|.  With RX[m] = max_k |x[m, k]| and RW[n] = max_k |w[n, k]| (attained at kx,
+// kw) the pair at kx shows out[m, n] >= RX[m] - RW[n], the pair at kw shows out[m, n] >= RW[n] - RX[m]; and inside a
+// 32-wide k-tile t no pair exceeds bx[m, t] + bw[n, t], the largest magnitudes of the two rows inside the tile.  So a
+// tile can hold the maximum of (m, n), or the first k that attains it, only if bx[m, t] + bw[n, t] reaches that lower
+// bound.  Two separable sufficient tests follow, with MX = max_m RX[m], MW = max_n RW[n] (per group):
+//   rows of x:  every tile with  bx[m, t] <  (RX[m] - MW) - MW  is dead for all n   (x decides: activations with few
+//               outliers against small weights)
+//   rows of w:  every tile with  bw[n, t] <  (RW[n] - MX) - MX  is dead for all m   (w decides: layers whose weights
+//               carry a large planted entry per row)
+// Either test alone is complete: under the first one no tile of w needs looking at beyond the tiles that are hot for
+// the row of x, and vice versa.  A pre-pass (shared with the k-tile skipping kernels) gives RX, RW and the tile
+// maxima; hot_plan_kernel turns them into one bit per (row, tile) for both tests, counts the bits and picks the
+// cheaper test, or neither when too many tiles are hot (then the dense kernels run: everything downstream is queued
+// gated on that decision, no host round trip).  inf_hot_kernel then walks, for every output, the hot tiles of its
+// owner row in ascending k with the reference's own comparison (strict "greater": the lowest k wins ties, NaN never
+// wins, 1e-10 floor with code 0), so values and codes need no second pass.
+// Rounding: the thresholds are evaluated in double with a relative margin of 2^-22, which covers the fp32 rounding
+// of the lower bound and of bx + bw (see hot_threshold).  A row that holds a NaN has a NaN row seed (the pair at its
+// kx may not exist then): all its tiles are hot, and if it is a row of the other side nothing is dead at all.
+#include <atomic>
+#include <stdlib.h>
+
+#include "ndist_common.h"
+
+namespace ndist {
+
+namespace {
+
+// Threshold below which a tile maximum of the owner row makes the tile dead: own = R of the owner row, other = the
+// largest R on the other side.  For a dead tile (b_own < A) and any row of the other side (b_other <= R_other <= other):
+//   b_own + b_other < A + other = (own - other)(1 - 2^-22) <= (own - R_other)(1 - 2^-22),
+// so fl32(b_own + b_other) <= (b_own + b_other)(1 + 2^-24) < (own - R_other)(1 - 2^-24) <= fl32(own - R_other) <= out:
+// strictly below the output, hence neither its value nor the first k attaining it.  (Sums and differences of two
+// floats are exact in the subnormal range, so the relative bounds hold there too.)  NaN (a row with a NaN, or
+// inf - inf) and own < other give "nothing is dead".
+__device__ __forceinline__ double hot_threshold(float own, float other) {
+    const double a = ((double)own - (double)other) * (1.0 - 0x1p-22) - (double)other;
+    return a == a ? a : -__builtin_inf();
+}
+
+// Largest row seed magnitude per group on both sides into LDS (sm[g] = MX, sm[G + g] = MW; infinite when a row of
+// that side holds a NaN), computed by every workgroup for itself: the arrays are a few thousand floats.
+__device__ __forceinline__ void hot_group_maxima(const float* __restrict__ seed_x, const float* __restrict__ seed_w,
+                                                 const Geom& s, unsigned* sm) {
+    for (int i = threadIdx.x; i < 2 * s.G; i += blockDim.x) sm[i] = 0u;
+    __syncthreads();
+    auto mag = [](float v) { v = fabsf(v); return v == v ? v : __builtin_inff(); };
+    // magnitudes are non-negative floats: their bit patterns order like unsigned integers
+    const long rows = (long)s.M * s.G, wrows = (long)s.COg * s.G;
+    const int lane = threadIdx.x & 63;
+    if (s.G == 1) {
+        float mx = 0.f, mw = 0.f;
+        for (long r = threadIdx.x; r < rows; r += blockDim.x) mx = fmaxf(mx, mag(seed_x[r]));
+        for (long r = threadIdx.x; r < wrows; r += blockDim.x) mw = fmaxf(mw, mag(seed_w[r]));
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) {
+            mx = fmaxf(mx, __shfl_xor(mx, d, 64));
+            mw = fmaxf(mw, __shfl_xor(mw, d, 64));
+        }
+        if (lane == 0) {
+            atomicMax(&sm[0], __float_as_uint(mx));
+            atomicMax(&sm[1], __float_as_uint(mw));
+        }
+    } else {
+        for (long r = threadIdx.x; r < rows; r += blockDim.x) atomicMax(&sm[r % s.G], __float_as_uint(mag(seed_x[r])));
+        for (long r = threadIdx.x; r < wrows; r += blockDim.x)
+            atomicMax(&sm[s.G + r / s.COg], __float_as_uint(mag(seed_w[r])));
+    }
+    __syncthreads();
+}
+
+// One kernel for the whole plan.  Every workgroup (1024 threads) first finds MX and MW of all groups, then its 16
+// waves turn 8 rows each (rows of x first, then rows of w) into hot-tile masks: bit t of a row's mask = tile t is
+// hot.  The workgroups leave their counts of hot (row, tile) entries per side in `partial`; the last one to finish
+// (a ticket in dec[3], cleared by the row pre-pass) adds them up and decides:
+//   dec[0] = 1: the rows of x select the tiles, 2: the rows of w, 0: too many hot tiles, the dense kernels run.
+// Cost of a side = its hot entries x the length of the other side.  mode: 1 always the cheaper side, 2 / 3 always
+// the x / w side, else the cheaper side if it touches at most 1 / frac of all (row, column, tile) triples.
+constexpr int kPlanRows = 128;
+__global__ __launch_bounds__(1024) void hot_plan_kernel(const float* __restrict__ seed_x, const float* __restrict__ seed_w,
+                                                        const float* __restrict__ tile_x, const float* __restrict__ tile_w,
+                                                        const Geom s, int ntile, int nword, uint32_t* __restrict__ mask_x,
+                                                        uint32_t* __restrict__ mask_w, int* __restrict__ dec,
+                                                        int* __restrict__ partial, int mode, int frac) {
+    extern __shared__ unsigned sm[];  // 2 * G maxima
+    __shared__ int cnt[2];
+    __shared__ int is_last;
+    __shared__ long long tot[2];
+    if (threadIdx.x < 2) { cnt[threadIdx.x] = 0; tot[threadIdx.x] = 0; }
+    hot_group_maxima(seed_x, seed_w, s, sm);
+    const long rows = (long)s.M * s.G, wrows = (long)s.COg * s.G;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int i = 0; i < kPlanRows / 16; i++) {
+        const long r = (long)blockIdx.x * kPlanRows + wave * (kPlanRows / 16) + i;
+        if (r >= rows + wrows) break;  // wave-uniform
+        const bool isw = r >= rows;
+        const long rr = isw ? r - rows : r;
+        const int g = isw ? (int)(rr / s.COg) : (int)(rr % s.G);
+        const float own = fabsf(isw ? seed_w[rr] : seed_x[rr]);
+        const double thr = hot_threshold(own, __uint_as_float(sm[isw ? g : s.G + g]));
+        const float* __restrict__ tm = (isw ? tile_w : tile_x) + rr * ntile;
+        uint32_t* __restrict__ mk = (isw ? mask_w : mask_x) + rr * nword;
+        int count = 0;
+        for (int t0 = 0; t0 < nword * 32; t0 += 64) {
+            const int t = t0 + lane;
+            const bool hot = t < ntile && !((double)tm[t] < thr);
+            const unsigned long long bits = __builtin_amdgcn_ballot_w64(hot);
+            count += __popcll(bits);
+            if (lane == 0) {
+                mk[t0 >> 5] = (uint32_t)bits;
+                if ((t0 >> 5) + 1 < nword) mk[(t0 >> 5) + 1] = (uint32_t)(bits >> 32);
+            }
+        }
+        if (lane == 0 && count != 0) atomicAdd(&cnt[isw ? 1 : 0], count);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        partial[2 * blockIdx.x] = cnt[0];
+        partial[2 * blockIdx.x + 1] = cnt[1];
+        __threadfence();  // the counts are visible device-wide before the ticket is taken
+        is_last = atomicAdd(&dec[3], 1) == (int)gridDim.x - 1;
+    }
+    __syncthreads();
+    if (!is_last) return;
+    __threadfence();
+    long long cx = 0, cw = 0;
+    for (int b = threadIdx.x; b < (int)gridDim.x; b += blockDim.x) {
+        cx += __atomic_load_n(&partial[2 * b], __ATOMIC_RELAXED);
+        cw += __atomic_load_n(&partial[2 * b + 1], __ATOMIC_RELAXED);
+    }
+    if (cx != 0) atomicAdd((unsigned long long*)&tot[0], (unsigned long long)cx);
+    if (cw != 0) atomicAdd((unsigned long long*)&tot[1], (unsigned long long)cw);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const long long costx = tot[0] * s.COg, costw = tot[1] * s.M;
+        const long long total = (long long)s.M * s.G * s.COg * ntile;
+        int choice = costx <= costw ? 1 : 2;
+        if (mode == 2) choice = 1;
+        else if (mode == 3) choice = 2;
+        else if (mode != 1 && (costx <= costw ? costx : costw) * frac > total) choice = 0;
+        dec[0] = choice;
+        dec[1] = (int)(tot[0] > 0x7fffffff ? 0x7fffffff : tot[0]);  // for inspection
+        dec[2] = (int)(tot[1] > 0x7fffffff ? 0x7fffffff : tot[1]);
+    }
+}
+
+template <bool TRACK>
+__device__ __forceinline__ void hot_pair(float xv, float wv, int k, float& best, uint32_t& code) {
+    const float d = xv - wv, a = fabsf(d);
+    if constexpr (TRACK) {
+        if (a > best) {
+            best = a;
+            code = (uint32_t)k | (d >= 0 ? 0u : kSignBit);
+        }
+    } else {
+        best = fmaxf(best, a);
+    }
+}
+
+// One wave: the hot tiles of one owner row (bits of mk, ascending k) against 64 rows of the other side.  Eight lanes
+// share a row of the other side and split a 32-wide tile into 16-byte pieces (a load instruction then covers eight
+// whole 128-byte rows instead of 64 different cache lines), lane group q of the wave serves the rows q, q + 8, ...,
+// q + 56 past `oth`, `stride` floats apart (`nrow` of them exist; the others re-read the first row and are
+// discarded by the caller).
+// X_OWNS: the owner is the row of x.  Every lane ends with the result of row 8 * (lane & 7) + (lane >> 3).
+template <bool TRACK, bool X_OWNS>
+__device__ __forceinline__ void hot_walk(const float* __restrict__ own, const float* __restrict__ oth, long stride,
+                                         int nrow, const uint32_t* __restrict__ mk, int nword, int K, bool vec,
+                                         float& best_out, uint32_t& code_out) {
+    const int lane = threadIdx.x & 63, sub = lane & 7, q = lane >> 3;
+    float best[8];
+    uint32_t code[8];
+    const float* rowp[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        best[j] = kEps;
+        code[j] = 0;
+        const int row = q + 8 * j;
+        rowp[j] = oth + (long)(row < nrow ? row : 0) * stride;
+    }
+    for (int wi = 0; wi < nword; wi++) {
+        uint32_t bits = mk[wi];
+        while (bits != 0) {
+            const int k0 = (wi * 32 + __builtin_ctz(bits)) * 32 + 4 * sub;
+            bits &= bits - 1;
+            if (vec && k0 + 4 <= K) {
+                const float4 o = *reinterpret_cast<const float4*>(own + k0);
+                float4 v[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) v[j] = *reinterpret_cast<const float4*>(rowp[j] + k0);
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    if constexpr (X_OWNS) {
+                        hot_pair<TRACK>(o.x, v[j].x, k0 + 0, best[j], code[j]);
+                        hot_pair<TRACK>(o.y, v[j].y, k0 + 1, best[j], code[j]);
+                        hot_pair<TRACK>(o.z, v[j].z, k0 + 2, best[j], code[j]);
+                        hot_pair<TRACK>(o.w, v[j].w, k0 + 3, best[j], code[j]);
+                    } else {
+                        hot_pair<TRACK>(v[j].x, o.x, k0 + 0, best[j], code[j]);
+                        hot_pair<TRACK>(v[j].y, o.y, k0 + 1, best[j], code[j]);
+                        hot_pair<TRACK>(v[j].z, o.z, k0 + 2, best[j], code[j]);
+                        hot_pair<TRACK>(v[j].w, o.w, k0 + 3, best[j], code[j]);
+                    }
+                }
+            } else {
+                const int k1 = min(k0 + 4, K);
+                for (int k = k0; k < k1; k++) {
+                    const float o = own[k];
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        if constexpr (X_OWNS) hot_pair<TRACK>(o, rowp[j][k], k, best[j], code[j]);
+                        else hot_pair<TRACK>(rowp[j][k], o, k, best[j], code[j]);
+                    }
+                }
+            }
+        }
+    }
+    // the eight lanes of a row merge: the larger value, among equal values the lower k ("nothing above the floor"
+    // is (1e-10, 0) in every lane that has it, so it never displaces a found pair and merges with itself)
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+#pragma unroll
+        for (int d = 1; d < 8; d <<= 1) {
+            const float ob = __shfl_xor(best[j], d, 64);
+            if constexpr (TRACK) {
+                const uint32_t oc = __shfl_xor(code[j], d, 64);
+                const bool take = ob > best[j] || (ob == best[j] && (oc & ~kSignBit) < (code[j] & ~kSignBit));
+                best[j] = take ? ob : best[j];
+                code[j] = take ? oc : code[j];
+            } else {
+                best[j] = fmaxf(best[j], ob);
+            }
+        }
+    }
+    best_out = best[0];
+    code_out = code[0];
+#pragma unroll
+    for (int j = 1; j < 8; j++) {
+        best_out = sub == j ? best[j] : best_out;
+        code_out = sub == j ? code[j] : code_out;
+    }
+}
+
+// The kernel that computes the outputs from the hot tiles, for whichever side the plan chose.
+//   dec[0] == 1, the rows of x own: a workgroup takes one row of x and 256 columns (64 per wave).
+//   dec[0] == 2, the rows of w own: a workgroup takes 16 rows of w (four per wave, one after the other) and 64 rows
+//   of x; the results turn around in LDS so that every row of the output is written 16 columns at a time.
+template <bool TRACK>
+__global__ __launch_bounds__(256) void inf_hot_kernel(const float* __restrict__ x, const float* __restrict__ w, const Geom s,
+                                                      const uint32_t* __restrict__ mask_x,
+                                                      const uint32_t* __restrict__ mask_w, int nword, int vec,
+                                                      float* __restrict__ out, int32_t* __restrict__ pos,
+                                                      const int* __restrict__ dec, unsigned grid_rows, unsigned grid_cols) {
+    __shared__ float tv[64][17];
+    __shared__ uint32_t tc[TRACK ? 64 : 1][17];
+    const int choice = dec[0];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int mine = 8 * (lane & 7) + (lane >> 3);  // the row of the other side whose result this lane ends up with
+    if (choice == 1) {
+        if (blockIdx.x >= grid_rows) return;
+        const int nchunk = ceil_div(s.COg, 256);
+        const long r = blockIdx.x / (unsigned)nchunk;  // row (m, g) of x
+        const int n0 = (int)(blockIdx.x % (unsigned)nchunk) * 256 + wave * 64;
+        if (n0 >= s.COg) return;  // whole waves
+        const int g = (int)(r % s.G);
+        float best;
+        uint32_t code;
+        hot_walk<TRACK, true>(x + r * s.CIg, w + ((long)g * s.COg + n0) * s.CIg, s.CIg, min(64, s.COg - n0),
+                              mask_x + r * nword, nword, s.CIg, vec != 0, best, code);
+        const int n = n0 + mine;
+        if (n < s.COg) {
+            out[r * s.COg + n] = best;
+            if constexpr (TRACK) pos[r * s.COg + n] = (int32_t)code;
+        }
+    } else if (choice == 2) {
+        if (blockIdx.x >= grid_cols) return;
+        const int nmb = ceil_div(s.M, 64), nnb = ceil_div(s.COg, 16);
+        unsigned id = blockIdx.x;
+        const int mb = (int)(id % (unsigned)nmb);
+        id /= (unsigned)nmb;
+        const int nb = (int)(id % (unsigned)nnb), g = (int)(id / (unsigned)nnb);
+        const int m0 = mb * 64;
+        // HW == 1: row m of group g of x starts at (m * G + g) * CIg, consecutive rows are G * CIg apart
+        for (int i = 0; i < 4; i++) {
+            const int c = wave * 4 + i, n = nb * 16 + c;
+            float best = kEps;
+            uint32_t code = 0;
+            if (n < s.COg) {  // wave-uniform
+                const long wrow = (long)g * s.COg + n;
+                hot_walk<TRACK, false>(w + wrow * s.CIg, x + ((long)m0 * s.G + g) * s.CIg, (long)s.CIg * s.G,
+                                       min(64, s.M - m0), mask_w + wrow * nword, nword, s.CIg, vec != 0, best, code);
+            }
+            tv[mine][c] = best;
+            if constexpr (TRACK) tc[mine][c] = code;
+        }
+        __syncthreads();
+        const int mr = threadIdx.x >> 2, mo = m0 + mr, c0 = (threadIdx.x & 3) * 4;
+        if (mo < s.M) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int n = nb * 16 + c0 + j;
+                if (n < s.COg) {
+                    const long o = ((long)mo * s.G + g) * s.COg + n;
+                    out[o] = tv[mr][c0 + j];
+                    if constexpr (TRACK) pos[o] = (int32_t)tc[mr][c0 + j];
+                }
+            }
+        }
+    }
+}
+
+int env_hot_mode() {
+    const char* v = getenv("NORM_DIST_HOT");
+    return v == nullptr || v[0] < '0' || v[0] > '3' ? -1 : v[0] - '0';
+}
+std::atomic<int> g_hot_mode{env_hot_mode()};
+
+}  // namespace
+
+void set_hot_mode(int mode) { g_hot_mode.store(mode < 0 || mode > 3 ? -1 : mode); }
+int hot_mode() { return g_hot_mode.load(); }
+
+static int plan_blocks(const Geom& s) {
+    return (int)(((long)s.M * s.G + (long)s.COg * s.G + kPlanRows - 1) / kPlanRows);
+}
+
+bool hot_forward_applies(const Geom& s) { return hot_mode() != 0 && s.HW == 1 && s.G <= 4096; }
+
+size_t hot_scratch_floats(const Geom& s) {
+    const size_t nword = (size_t)ceil_div(ceil_div(s.CIg, 32), 32);
+    return 8 + 2 * (size_t)plan_blocks(s) + nword * ((size_t)s.M * s.G + (size_t)s.COg * s.G);
+}
+
+int launch_inf_hot(const float* x, const float* w, const Geom& s, const SeedBuffers& sb, float* base, float* out,
+                   int32_t* pos, hipStream_t st, const int** decision) {
+    const int ntile = sb.ntile, nword = ceil_div(ntile, 32), nblk = plan_blocks(s);
+    const long rows = (long)s.M * s.G;
+    int* dec = reinterpret_cast<int*>(base);  // [0] decision, [1], [2] hot entries per side, [3] ticket (cleared by the row pre-pass)
+    int* partial = dec + 8;
+    uint32_t* mask_x = reinterpret_cast<uint32_t*>(partial + 2 * nblk);
+    uint32_t* mask_w = mask_x + rows * nword;
+    *decision = dec;
+    // at most 1 / 32 of all (row, column, tile) triples: beyond that the k-tile skipping dense kernel is the faster one
+    hipLaunchKernelGGL(hot_plan_kernel, dim3(nblk), dim3(1024), 2 * s.G * sizeof(unsigned), st, sb.seed_x, sb.seed_w,
+                       sb.tile_x, sb.tile_w, s, ntile, nword, mask_x, mask_w, dec, partial, hot_mode(), 32);
+    const int vec = s.CIg % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0;
+    const unsigned grid_r = (unsigned)(rows * ceil_div(s.COg, 256));
+    const unsigned grid_c = (unsigned)((long)ceil_div(s.M, 64) * ceil_div(s.COg, 16) * s.G);
+    const dim3 grid(grid_r > grid_c ? grid_r : grid_c);
+    if (pos != nullptr)
+        hipLaunchKernelGGL(inf_hot_kernel<true>, grid, dim3(256), 0, st, x, w, s, mask_x, mask_w, nword, vec, out, pos, dec,
+                           grid_r, grid_c);
+    else
+        hipLaunchKernelGGL(inf_hot_kernel<false>, grid, dim3(256), 0, st, x, w, s, mask_x, mask_w, nword, vec, out, pos, dec,
+                           grid_r, grid_c);
+    return hip_failed(hipGetLastError()) ? 4 : 0;
+}
+
+}  // namespace ndist

@@ -101,10 +101,10 @@ template <int KT>
 __global__ __launch_bounds__(256) void inf_rescan_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                          const float* __restrict__ out, int32_t* __restrict__ pos,
                                                          const Geom s, long total, int vec, int implicit,
-                                                         const PatchMap pm) {
+                                                         const PatchMap pm, const int* __restrict__ gate) {
     constexpr int kt = KT;
     const long o = (long)blockIdx.x * 256 + threadIdx.x;
-    if (o >= total) return;
+    if (o >= total || (gate != nullptr && gate[0] >= 1)) return;
     const int cid = pos[o];
     if (cid < 0) {  // nothing exceeded the floor
         pos[o] = 0;
@@ -164,46 +164,62 @@ int launch_inf_forward(const float* x, const float* w, const Geom& s, float* out
     // that skips the k-tiles which cannot matter (most of them, unless the largest |x - w| are far below
     // max|x| + max|w| everywhere).  NORM_DIST_SKIP=0 / ndist_set_skip_mode(0, ..) switches this off, 1 forces it on
     // for small problems too.
+    // Before those: from the same row pre-pass the hot-tile kernels (fwd_hot.hip) find out on the device whether
+    // few k-tiles decide all maxima; if so they produce the outputs themselves and everything queued below is gated off.
     const bool bounded = cv == nullptr && seeded_forward_applies(s);
+    const bool hot = bounded && hot_forward_applies(s);
     float* scratch = nullptr;
+    const int* gate = nullptr;
     KernelTimer timer(st);  // pre-passes + tiled kernel + rescan
     if (bounded) {
-        NDIST_HIP_TRY(scratch_alloc((void**)&scratch, seed_scratch_floats(s) * sizeof(float), st));
+        const size_t nseed = seed_scratch_floats(s);
+        NDIST_HIP_TRY(scratch_alloc((void**)&scratch, (nseed + (hot ? hot_scratch_floats(s) : 0)) * sizeof(float), st));
         SeedBuffers sb{};
-        const int rs = launch_seeds(x, w, s, scratch, nullptr, 0, st, &sb, nullptr, wpre);
+        int rs = launch_row_seeds(x, w, s, scratch, nullptr, 0, st, &sb, nullptr, wpre,
+                                  hot ? reinterpret_cast<int*>(scratch + nseed) : nullptr);
+        if (!rs && hot) rs = launch_inf_hot(x, w, s, sb, scratch + nseed, out, pos, st, &gate);
+        if (!rs) rs = launch_output_seeds(x, w, s, sb, gate, 1, st);
         if (rs) {
             (void)scratch_free(scratch, st);
             return rs;
+        }
+        if (gate != nullptr) {
+            P.gate = gate;
+            P.gate_limit = 1;
+            P.gate_sense = 1;
         }
         P.aux = sb.seed;
         P.tile_x = sb.tile_x;
         P.tile_w = sb.tile_w;
         P.ntile32 = sb.ntile;
     }
-    if (pos == nullptr) {
-        int rc = bounded ? launch_fwd<OpInf<false, true>, CfgWideT, CfgMid, CfgSmall>(P, st)
-                         : launch_fwd_conv<OpInf<false>, CfgWide4, CfgBig, CfgSmall, CfgWide>(P, st);
+    // (the scratch holds the gate: it is released after the last kernel that reads it has been queued)
+    auto done = [&](int rc) {
         if (bounded && hip_failed(scratch_free(scratch, st)) && !rc) rc = 4;
         return rc;
+    };
+    if (pos == nullptr) {
+        return done(bounded ? launch_fwd<OpInf<false, true>, CfgWideT, CfgMid, CfgSmall>(P, st)
+                            : launch_fwd_conv<OpInf<false>, CfgWide4, CfgBig, CfgSmall, CfgWide>(P, st));
     }
     int kt = 0;
-    int rc = bounded ? launch_fwd_layouts<false, OpInf<true, true>, CfgWideT, CfgMid, CfgSmall>(P, st, &kt)
-                     : launch_fwd_layouts<true, OpInf<true>, CfgWideT, CfgMid, CfgSmall>(P, st, &kt);
-    if (bounded && hip_failed(scratch_free(scratch, st)) && !rc) rc = 4;
-    if (rc) return rc;
-    if (rescan_sorted_applies(s, kt)) return launch_rescan_sorted<0>(x, nullptr, w, out, pos, s, kt, st, cv ? &pm : nullptr);
+    const int rc = bounded ? launch_fwd_layouts<false, OpInf<true, true>, CfgWideT, CfgMid, CfgSmall>(P, st, &kt)
+                           : launch_fwd_layouts<true, OpInf<true>, CfgWideT, CfgMid, CfgSmall>(P, st, &kt);
+    if (rc) return done(rc);
+    if (rescan_sorted_applies(s, kt))
+        return done(launch_rescan_sorted<0>(x, nullptr, w, out, pos, s, kt, st, cv ? &pm : nullptr));
     const long total = (long)s.M * s.COg * s.G;
     const int imp = cv != nullptr;
     const int vec = !imp && s.HW == 1 && s.CIg % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0;
     const dim3 grid((unsigned)((total + 255) / 256));
 #define NDIST_INF_RESCAN(KT_) \
-    hipLaunchKernelGGL(inf_rescan_kernel<KT_>, grid, dim3(256), 0, st, x, w, out, pos, s, total, vec, imp, pm)
+    hipLaunchKernelGGL(inf_rescan_kernel<KT_>, grid, dim3(256), 0, st, x, w, out, pos, s, total, vec, imp, pm, gate)
     if (kt == 4) NDIST_INF_RESCAN(4);
     else if (kt == 16) NDIST_INF_RESCAN(16);
     else if (kt == 32) NDIST_INF_RESCAN(32);
-    else return 2;
+    else return done(2);
 #undef NDIST_INF_RESCAN
-    return hip_failed(hipGetLastError()) ? 4 : 0;
+    return done(hip_failed(hipGetLastError()) ? 4 : 0);
 }
 
 }  // namespace ndist

@@ -425,31 +425,37 @@ __global__ __launch_bounds__(256) void norm_probe_count_kernel(const float* __re
 
 int fill_zero(float* p, long n, hipStream_t st);  // bwd_norm_c.hip
 
-// Pre-pass of the skipping operator over the rows of a matrix with k contiguous (x with HW == 1, or w), one wave per
-// row: the element of largest magnitude (signed) and its k, and the largest magnitude inside every 32-wide k-tile
-// (tile_max[row][ntile]).  Does nothing when the probe's count (gate[0]) says that the skipping operator will not run.
-__global__ __launch_bounds__(256) void norm_seed_kernel(const float* __restrict__ x, const float* __restrict__ x2,
-                                                        const Geom s,
-                                                        float* __restrict__ seed_x, int32_t* __restrict__ seed_k,
-                                                        float* __restrict__ tile_max, int ntile,
-                                                        const int* __restrict__ gate, int gate_limit) {
-    if (gate != nullptr && gate[0] >= gate_limit) return;
-    const long rows = (long)s.M * s.G;
-    const long r = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (r >= rows) return;  // whole waves leave: the shuffles below stay wave-uniform
+// Pre-pass of the skipping operators over the rows of a matrix with k contiguous (x with HW == 1, or w), one wave per
+// row: the element of largest magnitude (signed; NaN when the row holds a NaN) and its k, and the largest magnitude
+// inside every 32-wide k-tile (tile_max[row][ntile]).
+struct SeedSide {
+    const float* x;
+    const float* x2;  // interval bounds: second array of the same shape, the larger magnitude of the two counts
+    long rows;
+    int K;
+    float* seed;
+    int32_t* seed_k;
+    float* tile_max;
+};
+__device__ __forceinline__ void norm_seed_row(const SeedSide& sd, long r, int ntile) {
     const int lane = threadIdx.x & 63;
-    const float* __restrict__ xp = x + r * s.CIg;
-    const float* __restrict__ xq = x2 != nullptr ? x2 + r * s.CIg : nullptr;  // second array: magnitudes of both count
-    float* __restrict__ tm = tile_max + r * ntile;
+    const int K = sd.K;
+    const float* __restrict__ x = sd.x;
+    const float* __restrict__ xp = x + r * K;
+    const float* __restrict__ xq = sd.x2 != nullptr ? sd.x2 + r * K : nullptr;  // second array: magnitudes of both count
+    float* __restrict__ tm = sd.tile_max + r * ntile;
     float best = -1.f, val = 0.f;
     int bk = 0;
-    if (s.CIg % 4 == 0 && (uintptr_t)x % 16 == 0 && xq == nullptr) {  // 16-byte loads: 1 KiB per wave and iteration
-        for (int k0 = 0; k0 < s.CIg; k0 += 256) {
+    bool bad = false;  // a NaN in the row (or +inf next to -inf): the pair at the row's seed may not exist
+    if (K % 4 == 0 && (uintptr_t)x % 16 == 0 && xq == nullptr) {  // 16-byte loads: 1 KiB per wave and iteration
+        for (int k0 = 0; k0 < K; k0 += 256) {
             const int k = k0 + 4 * lane;
             float local = 0.f;  // largest magnitude of my four k: they lie in one tile, 8 lanes share a tile
-            if (k < s.CIg) {
+            if (k < K) {
                 const float4 v4 = *reinterpret_cast<const float4*>(xp + k);
                 const float v[4] = {v4.x, v4.y, v4.z, v4.w};
+                const float sum4 = (v4.x + v4.y) + (v4.z + v4.w);
+                bad |= sum4 != sum4;
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     local = fmaxf(local, fabsf(v[j]));
@@ -459,16 +465,18 @@ __global__ __launch_bounds__(256) void norm_seed_kernel(const float* __restrict_
             local = fmaxf(local, __shfl_xor(local, 1, 64));
             local = fmaxf(local, __shfl_xor(local, 2, 64));
             local = fmaxf(local, __shfl_xor(local, 4, 64));
-            if ((lane & 7) == 0 && k < s.CIg) tm[k >> 5] = local;
+            if ((lane & 7) == 0 && k < K) tm[k >> 5] = local;
         }
     } else {
-        for (int k0 = 0; k0 < s.CIg; k0 += 64) {
+        for (int k0 = 0; k0 < K; k0 += 64) {
             const int k = k0 + lane;
             float local = 0.f;  // 32 lanes share a tile
-            if (k < s.CIg) {
+            if (k < K) {
                 float v = xp[k];
+                bad |= v != v;
                 if (xq != nullptr) {
                     const float v2 = xq[k];
+                    bad |= v2 != v2;
                     v = fabsf(v2) > fabsf(v) ? v2 : v;
                 }
                 local = fabsf(v);
@@ -476,7 +484,7 @@ __global__ __launch_bounds__(256) void norm_seed_kernel(const float* __restrict_
             }
 #pragma unroll
             for (int d = 1; d < 32; d <<= 1) local = fmaxf(local, __shfl_xor(local, d, 64));
-            if ((lane & 31) == 0 && k < s.CIg) tm[k >> 5] = local;
+            if ((lane & 31) == 0 && k < K) tm[k >> 5] = local;
         }
     }
 #pragma unroll
@@ -485,7 +493,24 @@ __global__ __launch_bounds__(256) void norm_seed_kernel(const float* __restrict_
         const int ok = __shfl_xor(bk, d, 64);
         if (ob > best) { best = ob; val = ov; bk = ok; }
     }
-    if (lane == 0) { seed_x[r] = val; seed_k[r] = bk; }
+    // a row with a NaN is marked by a NaN seed value: consumers that form pairs with it drop them like any NaN pair
+    if (__builtin_amdgcn_ballot_w64(bad) != 0) val = __builtin_nanf("");
+    if (lane == 0) { sd.seed[r] = val; sd.seed_k[r] = bk; }
+}
+
+
+// Blocks [0, nblocks_a) serve side a, the others side b (four rows per block).  Does nothing when the probe's count
+// (gate[0]) says that the skipping operator will not run.  `zero`: four ints cleared for the kernels that follow.
+__global__ __launch_bounds__(256) void norm_seed_kernel(const SeedSide a, const SeedSide b, int nblocks_a, int ntile,
+                                                        const int* __restrict__ gate, int gate_limit,
+                                                        int* __restrict__ zero) {
+    if (zero != nullptr && blockIdx.x == 0 && threadIdx.x < 4) zero[threadIdx.x] = 0;
+    if (gate != nullptr && gate[0] >= gate_limit) return;
+    const bool second = (int)blockIdx.x >= nblocks_a;
+    const SeedSide& sd = second ? b : a;
+    const long r = (long)(blockIdx.x - (second ? nblocks_a : 0)) * 4 + (threadIdx.x >> 6);
+    if (r >= sd.rows) return;  // whole waves leave: the shuffles stay wave-uniform
+    norm_seed_row(sd, r, ntile);
 }
 
 // Seed of every output: the larger of the two pairs at the k of the row seeds of its x row and of its w row.
@@ -552,8 +577,10 @@ __global__ __launch_bounds__(256) void bound_seed_outputs_kernel(const float* __
                                                                  const float* __restrict__ seed_w,
                                                                  const int32_t* __restrict__ seed_wk,
                                                                  float* __restrict__ seed_hi, float* __restrict__ seed_lo,
-                                                                 int nmb, int nnb) {
+                                                                 int nmb, int nnb, const int* __restrict__ gate,
+                                                                 int gate_limit) {
     __shared__ float thi[64][65], tlo[64][65];
+    if (gate != nullptr && gate[0] >= gate_limit) return;
     unsigned id = blockIdx.x;
     const int nb = (int)(id % (unsigned)nnb);
     id /= (unsigned)nnb;
@@ -623,20 +650,14 @@ int launch_weight_seeds(const float* w, const Geom& s, float* base, const int* g
     out->seed_w = base;
     out->seed_wk = reinterpret_cast<int32_t*>(base + wrows);
     out->tile_w = reinterpret_cast<float*>(out->seed_wk + wrows);
-    // the rows of w: the row kernel on the geometry of a [CO, CIg] matrix
-    Geom ws{};
-    ws.B = ws.M = (int)wrows;
-    ws.HW = 1;
-    ws.G = 1;
-    ws.CIg = s.CIg;
-    ws.COg = 1;
-    hipLaunchKernelGGL(norm_seed_kernel, dim3((unsigned)((wrows + 3) / 4)), dim3(256), 0, st, w, (const float*)nullptr, ws,
-                       out->seed_w, out->seed_wk, out->tile_w, ntile, gate, gate_limit);
+    const SeedSide sw{w, nullptr, wrows, s.CIg, out->seed_w, out->seed_wk, out->tile_w};
+    hipLaunchKernelGGL(norm_seed_kernel, dim3((unsigned)((wrows + 3) / 4)), dim3(256), 0, st, sw, SeedSide{}, (int)((wrows + 3) / 4),
+                       ntile, gate, gate_limit, (int*)nullptr);
     return hip_failed(hipGetLastError()) ? 4 : 0;
 }
 
-int launch_seeds(const float* x, const float* w, const Geom& s, float* base, const int* gate, int gate_limit,
-                 hipStream_t st, SeedBuffers* out, const float* x2, const WeightSeeds* wpre) {
+int launch_row_seeds(const float* x, const float* w, const Geom& s, float* base, const int* gate, int gate_limit,
+                     hipStream_t st, SeedBuffers* out, const float* x2, const WeightSeeds* wpre, int* zero) {
     const long rows = (long)s.M * s.G, wrows = (long)s.COg * s.G, total = (long)s.M * s.COg * s.G;
     const int ntile = ceil_div(s.CIg, 32);
     int rc = 0;
@@ -648,42 +669,48 @@ int launch_seeds(const float* x, const float* w, const Geom& s, float* base, con
     float* tile_x = seed + total;
     float* tile_w = tile_x + rows * ntile;
     float* const after_tiles = tile_w + wrows * ntile;
-    hipLaunchKernelGGL(norm_seed_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, x, x2, s, seed_x, seed_k,
-                       tile_x, ntile, gate, gate_limit);
-    if (hip_failed(hipGetLastError())) rc = 4;
     if (wpre != nullptr) {
         seed_w = wpre->seed_w;
         seed_wk = wpre->seed_wk;
         tile_w = wpre->tile_w;
-    } else {
-        // the rows of w: the same kernel on the geometry of a [CO, CIg] matrix
-        Geom ws{};
-        ws.B = ws.M = (int)wrows;
-        ws.HW = 1;
-        ws.G = 1;
-        ws.CIg = s.CIg;
-        ws.COg = 1;
-        hipLaunchKernelGGL(norm_seed_kernel, dim3((unsigned)((wrows + 3) / 4)), dim3(256), 0, st, w, (const float*)nullptr,
-                           ws, seed_w, seed_wk, tile_w, ntile, gate, gate_limit);
-        if (hip_failed(hipGetLastError())) rc = 4;
     }
-    const int nmb = ceil_div(s.M, 64), nnb = ceil_div(s.COg, 64);
-    float* seed2 = nullptr;
-    if (x2 == nullptr) {
-        hipLaunchKernelGGL(norm_seed_outputs_kernel, dim3((unsigned)((long)nmb * nnb * s.G)), dim3(256), 0, st, x, w, s,
-                           seed_x, seed_k, seed_w, seed_wk, seed, nmb, nnb, gate, gate_limit);
-    } else {  // interval bounds (ungated): the second seed array lies behind the tile bounds
-        seed2 = after_tiles;
-        hipLaunchKernelGGL(bound_seed_outputs_kernel, dim3((unsigned)((long)nmb * nnb * s.G)), dim3(256), 0, st, x, x2, w,
-                           s, seed_k, seed_w, seed_wk, seed, seed2, nmb, nnb);
-    }
+    // one launch for the rows of x and (unless done before) the rows of w
+    const SeedSide sx{x, x2, rows, s.CIg, seed_x, seed_k, tile_x};
+    const SeedSide sw{w, nullptr, wpre != nullptr ? 0 : wrows, s.CIg, seed_w, seed_wk, tile_w};
+    const int nbx = (int)((rows + 3) / 4), nbw = (int)((sw.rows + 3) / 4);
+    hipLaunchKernelGGL(norm_seed_kernel, dim3((unsigned)(nbx + nbw)), dim3(256), 0, st, sx, sw, nbx, ntile, gate, gate_limit,
+                       zero);
     if (hip_failed(hipGetLastError())) rc = 4;
     out->seed = seed;
-    out->seed2 = seed2;
+    out->seed2 = x2 != nullptr ? after_tiles : nullptr;  // interval bounds: the second seed array lies behind the tile bounds
     out->tile_x = tile_x;
     out->tile_w = tile_w;
     out->ntile = ntile;
+    out->seed_x = seed_x;
+    out->seed_k = seed_k;
+    out->seed_w = seed_w;
+    out->seed_wk = seed_wk;
     return rc;
+}
+
+int launch_output_seeds(const float* x, const float* w, const Geom& s, const SeedBuffers& sb, const int* gate,
+                        int gate_limit, hipStream_t st, const float* x2) {
+    const int nmb = ceil_div(s.M, 64), nnb = ceil_div(s.COg, 64);
+    if (x2 == nullptr) {
+        hipLaunchKernelGGL(norm_seed_outputs_kernel, dim3((unsigned)((long)nmb * nnb * s.G)), dim3(256), 0, st, x, w, s,
+                           sb.seed_x, sb.seed_k, sb.seed_w, sb.seed_wk, sb.seed, nmb, nnb, gate, gate_limit);
+    } else {
+        hipLaunchKernelGGL(bound_seed_outputs_kernel, dim3((unsigned)((long)nmb * nnb * s.G)), dim3(256), 0, st, x, x2, w,
+                           s, sb.seed_k, sb.seed_w, sb.seed_wk, sb.seed, sb.seed2, nmb, nnb, gate, gate_limit);
+    }
+    return hip_failed(hipGetLastError()) ? 4 : 0;
+}
+
+int launch_seeds(const float* x, const float* w, const Geom& s, float* base, const int* gate, int gate_limit,
+                 hipStream_t st, SeedBuffers* out, const float* x2, const WeightSeeds* wpre) {
+    int rc = launch_row_seeds(x, w, s, base, gate, gate_limit, st, out, x2, wpre);
+    const int ro = launch_output_seeds(x, w, s, *out, gate, gate_limit, st, x2);
+    return rc ? rc : ro;
 }
 
 // Probe scratch: [0] the count (int), from float 4 on the maxima.  Zeroes it and leaves in [0] the number of sampled

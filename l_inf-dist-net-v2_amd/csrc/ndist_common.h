@@ -114,6 +114,11 @@ struct SeedBuffers {
     float* tile_x;
     float* tile_w;
     int ntile;
+    // per row of x / of w: the element of largest magnitude (NaN when the row holds a NaN) and its k
+    float* seed_x;
+    int32_t* seed_k;
+    float* seed_w;
+    int32_t* seed_wk;
 };
 // The part of the pre-passes that depends on w alone (per row of w: largest element, its k, tile maxima): two
 // operators called on the same weights (a layer's distance and its interval bounds) can share it.
@@ -129,6 +134,27 @@ int launch_weight_seeds(const float* w, const Geom& s, float* base, const int* g
 // `wpre`: weight rows already done by launch_weight_seeds (their part of `base` then stays unused)
 int launch_seeds(const float* x, const float* w, const Geom& s, float* base, const int* gate, int gate_limit,
                  hipStream_t st, SeedBuffers* out, const float* x2 = nullptr, const WeightSeeds* wpre = nullptr);
+// The two steps of launch_seeds: the row kernels (row seeds, tile bounds), then the seed of every output.
+// `zero`: four ints the row kernel clears on the way (counters of kernels queued behind it).
+int launch_row_seeds(const float* x, const float* w, const Geom& s, float* base, const int* gate, int gate_limit,
+                     hipStream_t st, SeedBuffers* out, const float* x2 = nullptr, const WeightSeeds* wpre = nullptr,
+                     int* zero = nullptr);
+int launch_output_seeds(const float* x, const float* w, const Geom& s, const SeedBuffers& sb, const int* gate,
+                        int gate_limit, hipStream_t st, const float* x2 = nullptr);
+
+// p = inf forward through hot k-tiles (fwd_hot.hip).  Queues the kernels that decide, from the row seeds and tile
+// bounds in `sb`, whether few enough k-tiles can hold the maxima, and the kernels that then compute out (and pos
+// unless null) from those tiles alone.  *decision points at an int that is 0 on the device when they did not run:
+// the caller queues the dense kernels gated on it (run while decision[0] < 1).  `base`: hot_scratch_floats(s) floats.
+// Mode (ndist_set_hot_mode / NORM_DIST_HOT): -1 the counts decide, 0 off, 1 always the cheaper side, 2 / 3 always the
+// rows of x / of w.
+// `base` starts with the four ints the row pre-pass has to clear (launch_row_seeds' `zero`).
+bool hot_forward_applies(const Geom& s);
+size_t hot_scratch_floats(const Geom& s);
+int launch_inf_hot(const float* x, const float* w, const Geom& s, const SeedBuffers& sb, float* base, float* out,
+                   int32_t* pos, hipStream_t st, const int** decision);
+void set_hot_mode(int mode);
+int hot_mode();
 
 #define NDIST_HIP_TRY(expr)                                        \
     do {                                                           \

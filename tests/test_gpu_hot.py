@@ -1,0 +1,88 @@
+"""p = inf forward through hot k-tiles (reference: core/cuda/inf_dist_cuda.cu:14-198,248-317): on data where a few
+k decide every maximum the library computes the outputs from those k-tiles alone.  Values and arg-max codes must be
+bit-identical to the oracle whichever side (rows of x, rows of w) selects the tiles, also when the selection is
+forced onto data it would not be chosen for (then nearly every tile is hot), with ties, floors, NaN, infinities,
+groups and ragged sizes.  ndist_set_skip_mode(1, .) makes the seeded paths serve these small shapes,
+ndist_set_hot_mode picks the side."""
+import numpy as np
+import pytest
+
+from oracle import norm_dist_oracle as O
+from util import gpu_inf_forward
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [  # B, CO, CI, G
+    (37, 50, 333, 1),      # ragged everything, scalar loads
+    (200, 300, 1024, 1),   # full tiles, 16-byte loads
+    (130, 96, 1056, 2),    # two groups, a last partial 64-tile word
+    (64, 16, 4100, 1),     # more than 128 tiles: masks of five words, partial last tile
+    (5, 700, 96, 1),       # few rows, many columns
+]
+
+
+@pytest.fixture
+def modes():
+    from core import _C
+    _C.set_skip_mode(1, -1)
+    yield _C.set_hot_mode
+    _C.set_hot_mode(-1)
+    _C.set_skip_mode(-1, -1)
+
+
+def _data(kind, B, CO, CI, G, seed):
+    r = np.random.RandomState(seed)
+    K = CI // G
+    x = r.randn(B, CI, 1).astype(np.float32)
+    w = r.randn(CO, K).astype(np.float32)
+    if kind == "small_w":        # the outliers of x decide
+        w /= np.sqrt(K)
+    elif kind == "diagonal":     # a planted entry per row of w decides
+        w *= 0.3
+        for n in range(CO):
+            w[n, n % K] = -10.0
+    elif kind == "ties":         # small integers: many equal maxima, the lowest k must win
+        x = r.randint(-3, 4, size=x.shape).astype(np.float32)
+        w = r.randint(-3, 4, size=w.shape).astype(np.float32)
+    elif kind == "floor":        # every difference at or below the 1e-10 floor: value 1e-10, code 0
+        x = np.repeat(r.randn(1, CI, 1).astype(np.float32), B, axis=0)
+        w = np.concatenate([np.tile(x[0, g * K:(g + 1) * K, 0], (CO // G, 1)) for g in range(G)])
+        w = np.ascontiguousarray(w, dtype=np.float32)
+    elif kind == "special":      # NaN and infinities in both operands
+        w /= np.sqrt(K)
+        x[1, 5, 0] = np.nan
+        x[2, 7 % CI, 0] = np.inf
+        x[3, 9 % CI, 0] = -np.inf
+        x[3, 10 % CI, 0] = np.inf
+        w[2, 3] = np.nan
+        w[4 % CO, 11 % K] = np.inf
+        w[5 % CO, 7 % K] = np.inf   # inf - inf against x[2]
+    return x, w
+
+
+@pytest.mark.parametrize("mode", [2, 3, 1, -1, 0])
+@pytest.mark.parametrize("kind", ["small_w", "diagonal", "normal", "ties", "floor", "special"])
+@pytest.mark.parametrize("B,CO,CI,G", SHAPES)
+def test_hot_tiles_match_the_oracle(modes, B, CO, CI, G, kind, mode):
+    if kind == "floor" and CO % G:
+        pytest.skip("needs whole groups")
+    modes(mode)
+    x, w = _data(kind, B, CO, CI, G, seed=B + CO)
+    eo, ep = O.inf_dist_forward(x, w, G)
+    out, pos = gpu_inf_forward(x, w, G)
+    assert np.array_equal(out.view(np.uint32), eo.view(np.uint32)), "values %s mode %d" % (kind, mode)
+    assert np.array_equal(pos, ep), "codes %s mode %d" % (kind, mode)
+    out2, _ = gpu_inf_forward(x, w, G, with_pos=False)
+    assert np.array_equal(out2.view(np.uint32), eo.view(np.uint32)), "values without codes %s mode %d" % (kind, mode)
+
+
+def test_decision_follows_the_data(modes):
+    """With the counts deciding, both kinds of sparse data and dense data give the oracle's bits at a size where the
+    choice matters (the kernel names in a profile tell which path ran; here only the results are checked)."""
+    modes(-1)
+    B, CO, CI = 256, 1024, 2048
+    for kind in ("small_w", "diagonal", "normal"):
+        x, w = _data(kind, B, CO, CI, 1, seed=11)
+        eo, ep = O.inf_dist_forward(x, w)
+        out, pos = gpu_inf_forward(x, w)
+        assert np.array_equal(out, eo) and np.array_equal(pos, ep), kind
