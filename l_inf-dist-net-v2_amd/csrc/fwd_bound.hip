@@ -111,9 +111,10 @@ __global__ __launch_bounds__(256) void bound_rescan_kernel(const float* __restri
                                                            const float* __restrict__ w, const float* __restrict__ yl,
                                                            const float* __restrict__ yu, int32_t* __restrict__ posl,
                                                            int32_t* __restrict__ posu, const Geom s, long total, int vec,
-                                                           int implicit, const PatchMap pm) {
+                                                           int implicit, const PatchMap pm,
+                                                           const int* __restrict__ gate) {
     const long o = (long)blockIdx.x * 256 + threadIdx.x;
-    if (o >= total) return;
+    if (o >= total || (gate != nullptr && gate[0] >= 1)) return;
     const int hw = (int)(o % s.HW);
     const long r = o / s.HW;
     const int gco = (int)(r % (s.COg * s.G));
@@ -180,19 +181,29 @@ int launch_bound_forward(const float* xl, const float* xu, const float* w, const
     P.pos = pl;
     P.pos2 = pu;
     P.s = s;
-    // large fully-connected problems: seeds and k-tile bounds, as in launch_inf_forward
+    // large fully-connected problems: hot-tile kernels first, else seeds and k-tile bounds, as in launch_inf_forward
     const bool bounded = cv == nullptr && seeded_forward_applies(s);
     if (!bounded && pl == nullptr) return launch_fwd_conv<OpBound<false>, CfgBoundN, CfgMid, CfgSmall>(P, st);
+    const bool hot = bounded && hot_forward_applies(s);
     KernelTimer timer(st);  // pre-passes + tiled kernel + rescan
     float* scratch = nullptr;
+    const int* gate = nullptr;
     if (bounded) {
-        const size_t total = (size_t)s.M * s.COg * s.G;
-        NDIST_HIP_TRY(scratch_alloc((void**)&scratch, (seed_scratch_floats(s) + total) * sizeof(float), st));
+        const size_t nseed = bound_seed_scratch_floats(s);
+        NDIST_HIP_TRY(scratch_alloc((void**)&scratch, (nseed + (hot ? hot_scratch_floats(s) : 0)) * sizeof(float), st));
         SeedBuffers sb{};
-        const int rs = launch_seeds(xl, w, s, scratch, nullptr, 0, st, &sb, xu, wpre);
+        int rs = launch_row_seeds(xl, w, s, scratch, nullptr, 0, st, &sb, xu, wpre,
+                                  hot ? reinterpret_cast<int*>(scratch + nseed) : nullptr);
+        if (!rs && hot) rs = launch_bound_hot(xl, xu, w, s, sb, scratch + nseed, yl, yu, pl, pu, st, &gate);
+        if (!rs) rs = launch_output_seeds(xl, w, s, sb, gate, 1, st, xu);
         if (rs) {
             (void)scratch_free(scratch, st);
             return rs;
+        }
+        if (gate != nullptr) {
+            P.gate = gate;
+            P.gate_limit = 1;
+            P.gate_sense = 1;
         }
         P.aux = sb.seed;
         P.aux2 = sb.seed2;
@@ -200,33 +211,33 @@ int launch_bound_forward(const float* xl, const float* xu, const float* w, const
         P.tile_w = sb.tile_w;
         P.ntile32 = sb.ntile;
     }
-    if (pl == nullptr) {
-        int rc = launch_fwd<OpBound<false, true>, CfgBoundT, CfgMid, CfgSmall>(P, st);
-        if (hip_failed(scratch_free(scratch, st)) && !rc) rc = 4;
+    // (the scratch holds the gate: it is released after the last kernel that reads it has been queued)
+    auto done = [&](int rc) {
+        if (bounded && hip_failed(scratch_free(scratch, st)) && !rc) rc = 4;
         return rc;
-    }
+    };
+    if (pl == nullptr) return done(launch_fwd<OpBound<false, true>, CfgBoundT, CfgMid, CfgSmall>(P, st));
     int kt = 0;
-    int rc = bounded ? launch_fwd_layouts<false, OpBound<true, true>, CfgBoundT, CfgSmall>(P, st, &kt)
-                     : launch_fwd_layouts<true, OpBound<true>, CfgBoundT, CfgSmall>(P, st, &kt);
-    if (bounded && hip_failed(scratch_free(scratch, st)) && !rc) rc = 4;
-    if (rc) return rc;
+    const int rc = bounded ? launch_fwd_layouts<false, OpBound<true, true>, CfgBoundT, CfgSmall>(P, st, &kt)
+                           : launch_fwd_layouts<true, OpBound<true>, CfgBoundT, CfgSmall>(P, st, &kt);
+    if (rc) return done(rc);
     const int imp = cv != nullptr;
     if (rescan_sorted_applies(s, kt)) {
         const int r1 = launch_rescan_sorted<1>(xl, xu, w, yl, pl, s, kt, st, imp ? &pm : nullptr);
-        return r1 ? r1 : launch_rescan_sorted<2>(xl, xu, w, yu, pu, s, kt, st, imp ? &pm : nullptr);
+        return done(r1 ? r1 : launch_rescan_sorted<2>(xl, xu, w, yu, pu, s, kt, st, imp ? &pm : nullptr));
     }
     const long total = (long)s.M * s.COg * s.G;
     const int vec = !imp && s.HW == 1 && s.CIg % 4 == 0 && (uintptr_t)xl % 16 == 0 && (uintptr_t)xu % 16 == 0 &&
                     (uintptr_t)w % 16 == 0;
     const dim3 grid((unsigned)((total + 255) / 256));
 #define NDIST_BOUND_RESCAN(KT_) \
-    hipLaunchKernelGGL(bound_rescan_kernel<KT_>, grid, dim3(256), 0, st, xl, xu, w, yl, yu, pl, pu, s, total, vec, imp, pm)
+    hipLaunchKernelGGL(bound_rescan_kernel<KT_>, grid, dim3(256), 0, st, xl, xu, w, yl, yu, pl, pu, s, total, vec, imp, pm, gate)
     if (kt == 4) NDIST_BOUND_RESCAN(4);
     else if (kt == 16) NDIST_BOUND_RESCAN(16);
     else if (kt == 32) NDIST_BOUND_RESCAN(32);
-    else return 2;
+    else return done(2);
 #undef NDIST_BOUND_RESCAN
-    return hip_failed(hipGetLastError()) ? 4 : 0;
+    return done(hip_failed(hipGetLastError()) ? 4 : 0);
 }
 
 // A layer's distance and its interval bounds in one call (certification runs both on every layer with the same

@@ -74,18 +74,20 @@ __device__ __forceinline__ void hot_group_maxima(const float* __restrict__ seed_
 }
 
 // One kernel for the whole plan.  Every workgroup (1024 threads) first finds MX and MW of all groups, then its 16
-// waves turn 8 rows each (rows of x first, then rows of w) into hot-tile masks: bit t of a row's mask = tile t is
+// waves turn one row each (rows of x first, then rows of w) into hot-tile masks: bit t of a row's mask = tile t is
 // hot.  The workgroups leave their counts of hot (row, tile) entries per side in `partial`; the last one to finish
 // (a ticket in dec[3], cleared by the row pre-pass) adds them up and decides:
 //   dec[0] = 1: the rows of x select the tiles, 2: the rows of w, 0: too many hot tiles, the dense kernels run.
 // Cost of a side = its hot entries x the length of the other side.  mode: 1 always the cheaper side, 2 / 3 always
 // the x / w side, else the cheaper side if it touches at most 1 / frac of all (row, column, tile) triples.
-constexpr int kPlanRows = 128;
+constexpr int kPlanRows = 16;  // one row per wave: the chain of dependent loads per wave stays short
 __global__ __launch_bounds__(1024) void hot_plan_kernel(const float* __restrict__ seed_x, const float* __restrict__ seed_w,
                                                         const float* __restrict__ tile_x, const float* __restrict__ tile_w,
                                                         const Geom s, int ntile, int nword, uint32_t* __restrict__ mask_x,
                                                         uint32_t* __restrict__ mask_w, int* __restrict__ dec,
-                                                        int* __restrict__ partial, int mode, int frac) {
+                                                        int* __restrict__ partial, int mode, int frac,
+                                                        const float* __restrict__ far_hi,
+                                                        const float* __restrict__ far_lo) {
     extern __shared__ unsigned sm[];  // 2 * G maxima
     __shared__ int cnt[2];
     __shared__ int is_last;
@@ -101,7 +103,14 @@ __global__ __launch_bounds__(1024) void hot_plan_kernel(const float* __restrict_
         const long rr = isw ? r - rows : r;
         const int g = isw ? (int)(rr / s.COg) : (int)(rr % s.G);
         const float own = fabsf(isw ? seed_w[rr] : seed_x[rr]);
-        const double thr = hot_threshold(own, __uint_as_float(sm[isw ? g : s.G + g]));
+        const float other = __uint_as_float(sm[isw ? g : s.G + g]);
+        double thr = hot_threshold(own, other);
+        if (!isw && far_hi != nullptr) {
+            // interval bounds, rows of the box: the two reductions have their own lower bounds, far_hi - RW for the
+            // upper one and far_lo - RW for the lower one; a tile is dead when it is dead for both
+            const double tu = hot_threshold(far_hi[rr], other), tl = hot_threshold(far_lo[rr], other);
+            thr = own == own ? (tu < tl ? tu : tl) : -__builtin_inf();
+        }
         const float* __restrict__ tm = (isw ? tile_w : tile_x) + rr * ntile;
         uint32_t* __restrict__ mk = (isw ? mask_w : mask_x) + rr * nword;
         int count = 0;
@@ -148,37 +157,107 @@ __global__ __launch_bounds__(1024) void hot_plan_kernel(const float* __restrict_
     }
 }
 
+// The two operators as policies of the walk: per-output state, one pair, the merge of two lanes' states (the larger
+// value, among equal values the lower k; "nothing found" carries the operator's initial code, which no found pair
+// can tie with because a pair must beat the floor strictly), the outputs.
 template <bool TRACK>
-__device__ __forceinline__ void hot_pair(float xv, float wv, int k, float& best, uint32_t& code) {
-    const float d = xv - wv, a = fabsf(d);
-    if constexpr (TRACK) {
-        if (a > best) {
-            best = a;
-            code = (uint32_t)k | (d >= 0 ? 0u : kSignBit);
+struct HotInf {  // out = max(1e-10, max_k |x - w|), code = k | sign flag (core/cuda/inf_dist_cuda.cu:131-132,173-177)
+    static constexpr int NX = 1, NF = 1, NI = TRACK ? 1 : 0;
+    struct State { float best; uint32_t code; };
+    __device__ static __forceinline__ void init(State& a) { a.best = kEps; a.code = 0; }
+    __device__ static __forceinline__ void pair(State& a, float xv, float, float wv, int k) {
+        const float d = xv - wv, v = fabsf(d);
+        if constexpr (TRACK) {
+            if (v > a.best) { a.best = v; a.code = (uint32_t)k | (d >= 0 ? 0u : kSignBit); }
+        } else {
+            a.best = fmaxf(a.best, v);
         }
-    } else {
-        best = fmaxf(best, a);
     }
-}
+    __device__ static __forceinline__ void merge_xor(State& a, int d) {
+        const float ob = __shfl_xor(a.best, d, 64);
+        if constexpr (TRACK) {
+            const uint32_t oc = __shfl_xor(a.code, d, 64);
+            const bool take = ob > a.best || (ob == a.best && (oc & ~kSignBit) < (a.code & ~kSignBit));
+            a.best = take ? ob : a.best;
+            a.code = take ? oc : a.code;
+        } else {
+            a.best = fmaxf(a.best, ob);
+        }
+    }
+    __device__ static __forceinline__ void select(State& a, const State& b, bool c) {
+        a.best = c ? b.best : a.best;
+        a.code = c ? b.code : a.code;
+    }
+    __device__ static __forceinline__ void outputs(const State& a, float* f, uint32_t* i) {
+        f[0] = a.best;
+        if constexpr (TRACK) i[0] = a.code;
+    }
+};
+
+template <bool TRACK>
+struct HotBound {  // interval bounds (core/cuda/bound_inf_dist_cuda.cu:63,148-151,203-213,225-232)
+    static constexpr int NX = 2, NF = 2, NI = TRACK ? 2 : 0;
+    struct State { float lo, hi; uint32_t wl, wu; };
+    __device__ static __forceinline__ void init(State& a) { a.lo = -kEps; a.hi = kEps; a.wl = kNoGradId; a.wu = 0; }
+    __device__ static __forceinline__ void pair(State& a, float xl, float xu, float wv, int k) {
+        if (xl > xu) xl = xu = (xl + xu) * 0.5f;  // an inverted box collapses to its midpoint
+        const float t1 = wv - xl, t2 = xu - wv;
+        const float mn = fminf(t1, t2), mx = fmaxf(t1, t2);
+        if constexpr (TRACK) {
+            const uint32_t code = (uint32_t)k | (t1 <= t2 ? 0u : kSignBit);
+            if (mn < a.lo) { a.lo = mn; a.wl = code; }
+            if (mx > a.hi) { a.hi = mx; a.wu = code; }
+        } else {
+            a.lo = fminf(a.lo, mn);
+            a.hi = fmaxf(a.hi, mx);
+        }
+    }
+    __device__ static __forceinline__ void merge_xor(State& a, int d) {
+        const float ol = __shfl_xor(a.lo, d, 64), oh = __shfl_xor(a.hi, d, 64);
+        if constexpr (TRACK) {
+            const uint32_t cl = __shfl_xor(a.wl, d, 64), cu = __shfl_xor(a.wu, d, 64);
+            const bool tl = ol < a.lo || (ol == a.lo && (cl & ~kSignBit) < (a.wl & ~kSignBit));
+            const bool tu = oh > a.hi || (oh == a.hi && (cu & ~kSignBit) < (a.wu & ~kSignBit));
+            a.lo = tl ? ol : a.lo;
+            a.wl = tl ? cl : a.wl;
+            a.hi = tu ? oh : a.hi;
+            a.wu = tu ? cu : a.wu;
+        } else {
+            a.lo = fminf(a.lo, ol);
+            a.hi = fmaxf(a.hi, oh);
+        }
+    }
+    __device__ static __forceinline__ void select(State& a, const State& b, bool c) {
+        a.lo = c ? b.lo : a.lo;
+        a.hi = c ? b.hi : a.hi;
+        a.wl = c ? b.wl : a.wl;
+        a.wu = c ? b.wu : a.wu;
+    }
+    __device__ static __forceinline__ void outputs(const State& a, float* f, uint32_t* i) {
+        f[0] = -a.lo;
+        f[1] = a.hi;
+        if constexpr (TRACK) { i[0] = a.wl; i[1] = a.wu; }
+    }
+};
 
 // One wave: the hot tiles of one owner row (bits of mk, ascending k) against 64 rows of the other side.  Eight lanes
 // share a row of the other side and split a 32-wide tile into 16-byte pieces (a load instruction then covers eight
 // whole 128-byte rows instead of 64 different cache lines), lane group q of the wave serves the rows q, q + 8, ...,
 // q + 56 past `oth`, `stride` floats apart (`nrow` of them exist; the others re-read the first row and are
-// discarded by the caller).
-// X_OWNS: the owner is the row of x.  Every lane ends with the result of row 8 * (lane & 7) + (lane >> 3).
-template <bool TRACK, bool X_OWNS>
-__device__ __forceinline__ void hot_walk(const float* __restrict__ own, const float* __restrict__ oth, long stride,
-                                         int nrow, const uint32_t* __restrict__ mk, int nword, int K, bool vec,
-                                         float& best_out, uint32_t& code_out) {
+// discarded by the caller).  X_OWNS: the owner is the row of x.  x has a second array at distance `x2off` floats
+// for the interval bounds (P::NX == 2).  Every lane ends with the result of row 8 * (lane & 7) + (lane >> 3).
+template <class P, bool X_OWNS>
+__device__ __forceinline__ void hot_walk(const float* __restrict__ own, const float* __restrict__ oth, long x2off,
+                                         long stride, int nrow, const uint32_t* __restrict__ mk, int nword, int K,
+                                         bool vec, typename P::State& res) {
+    using State = typename P::State;
+    constexpr bool TWO = P::NX == 2;
     const int lane = threadIdx.x & 63, sub = lane & 7, q = lane >> 3;
-    float best[8];
-    uint32_t code[8];
+    State st[8];
     const float* rowp[8];
 #pragma unroll
     for (int j = 0; j < 8; j++) {
-        best[j] = kEps;
-        code[j] = 0;
+        P::init(st[j]);
         const int row = q + 8 * j;
         rowp[j] = oth + (long)(row < nrow ? row : 0) * stride;
     }
@@ -189,77 +268,77 @@ __device__ __forceinline__ void hot_walk(const float* __restrict__ own, const fl
             bits &= bits - 1;
             if (vec && k0 + 4 <= K) {
                 const float4 o = *reinterpret_cast<const float4*>(own + k0);
-                float4 v[8];
+                float4 o2 = o;
+                if constexpr (TWO && X_OWNS) o2 = *reinterpret_cast<const float4*>(own + x2off + k0);
+                float4 v[8], v2[TWO && !X_OWNS ? 8 : 1];
 #pragma unroll
-                for (int j = 0; j < 8; j++) v[j] = *reinterpret_cast<const float4*>(rowp[j] + k0);
+                for (int j = 0; j < 8; j++) {
+                    v[j] = *reinterpret_cast<const float4*>(rowp[j] + k0);
+                    if constexpr (TWO && !X_OWNS) v2[j] = *reinterpret_cast<const float4*>(rowp[j] + x2off + k0);
+                }
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
                     if constexpr (X_OWNS) {
-                        hot_pair<TRACK>(o.x, v[j].x, k0 + 0, best[j], code[j]);
-                        hot_pair<TRACK>(o.y, v[j].y, k0 + 1, best[j], code[j]);
-                        hot_pair<TRACK>(o.z, v[j].z, k0 + 2, best[j], code[j]);
-                        hot_pair<TRACK>(o.w, v[j].w, k0 + 3, best[j], code[j]);
+                        P::pair(st[j], o.x, o2.x, v[j].x, k0 + 0);
+                        P::pair(st[j], o.y, o2.y, v[j].y, k0 + 1);
+                        P::pair(st[j], o.z, o2.z, v[j].z, k0 + 2);
+                        P::pair(st[j], o.w, o2.w, v[j].w, k0 + 3);
                     } else {
-                        hot_pair<TRACK>(v[j].x, o.x, k0 + 0, best[j], code[j]);
-                        hot_pair<TRACK>(v[j].y, o.y, k0 + 1, best[j], code[j]);
-                        hot_pair<TRACK>(v[j].z, o.z, k0 + 2, best[j], code[j]);
-                        hot_pair<TRACK>(v[j].w, o.w, k0 + 3, best[j], code[j]);
+                        const float4 u = TWO ? v2[TWO && !X_OWNS ? j : 0] : v[j];
+                        P::pair(st[j], v[j].x, u.x, o.x, k0 + 0);
+                        P::pair(st[j], v[j].y, u.y, o.y, k0 + 1);
+                        P::pair(st[j], v[j].z, u.z, o.z, k0 + 2);
+                        P::pair(st[j], v[j].w, u.w, o.w, k0 + 3);
                     }
                 }
             } else {
                 const int k1 = min(k0 + 4, K);
                 for (int k = k0; k < k1; k++) {
-                    const float o = own[k];
+                    const float o = own[k], o2 = TWO && X_OWNS ? own[x2off + k] : o;
 #pragma unroll
                     for (int j = 0; j < 8; j++) {
-                        if constexpr (X_OWNS) hot_pair<TRACK>(o, rowp[j][k], k, best[j], code[j]);
-                        else hot_pair<TRACK>(rowp[j][k], o, k, best[j], code[j]);
+                        if constexpr (X_OWNS) P::pair(st[j], o, o2, rowp[j][k], k);
+                        else P::pair(st[j], rowp[j][k], TWO ? rowp[j][x2off + k] : 0.f, o, k);
                     }
                 }
             }
         }
     }
-    // the eight lanes of a row merge: the larger value, among equal values the lower k ("nothing above the floor"
-    // is (1e-10, 0) in every lane that has it, so it never displaces a found pair and merges with itself)
+    // the eight lanes of a row merge
 #pragma unroll
     for (int j = 0; j < 8; j++) {
 #pragma unroll
-        for (int d = 1; d < 8; d <<= 1) {
-            const float ob = __shfl_xor(best[j], d, 64);
-            if constexpr (TRACK) {
-                const uint32_t oc = __shfl_xor(code[j], d, 64);
-                const bool take = ob > best[j] || (ob == best[j] && (oc & ~kSignBit) < (code[j] & ~kSignBit));
-                best[j] = take ? ob : best[j];
-                code[j] = take ? oc : code[j];
-            } else {
-                best[j] = fmaxf(best[j], ob);
-            }
-        }
+        for (int d = 1; d < 8; d <<= 1) P::merge_xor(st[j], d);
     }
-    best_out = best[0];
-    code_out = code[0];
+    res = st[0];
 #pragma unroll
-    for (int j = 1; j < 8; j++) {
-        best_out = sub == j ? best[j] : best_out;
-        code_out = sub == j ? code[j] : code_out;
-    }
+    for (int j = 1; j < 8; j++) P::select(res, st[j], sub == j);
 }
+
+struct HotOut {
+    float* f[2];
+    int32_t* i[2];
+};
 
 // The kernel that computes the outputs from the hot tiles, for whichever side the plan chose.
 //   dec[0] == 1, the rows of x own: a workgroup takes one row of x and 256 columns (64 per wave).
 //   dec[0] == 2, the rows of w own: a workgroup takes 16 rows of w (four per wave, one after the other) and 64 rows
 //   of x; the results turn around in LDS so that every row of the output is written 16 columns at a time.
-template <bool TRACK>
-__global__ __launch_bounds__(256) void inf_hot_kernel(const float* __restrict__ x, const float* __restrict__ w, const Geom s,
-                                                      const uint32_t* __restrict__ mask_x,
-                                                      const uint32_t* __restrict__ mask_w, int nword, int vec,
-                                                      float* __restrict__ out, int32_t* __restrict__ pos,
-                                                      const int* __restrict__ dec, unsigned grid_rows, unsigned grid_cols) {
-    __shared__ float tv[64][17];
-    __shared__ uint32_t tc[TRACK ? 64 : 1][17];
+// x2off: distance in floats from x (the lower input bound) to the upper one (interval bounds only).
+template <class P>
+__global__ __launch_bounds__(256) void hot_kernel(const float* __restrict__ x, long x2off, const float* __restrict__ w,
+                                                  const Geom s, const uint32_t* __restrict__ mask_x,
+                                                  const uint32_t* __restrict__ mask_w, int nword, int vec, const HotOut out,
+                                                  const int* __restrict__ dec, unsigned grid_rows, unsigned grid_cols) {
+    constexpr int NF = P::NF, NI = P::NI;
+    __shared__ float tv[NF][64][17];
+    __shared__ uint32_t tc[NI > 0 ? NI : 1][64][17];
     const int choice = dec[0];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int mine = 8 * (lane & 7) + (lane >> 3);  // the row of the other side whose result this lane ends up with
+    typename P::State res;
+    float fv[NF];
+    uint32_t iv[NI > 0 ? NI : 1];
     if (choice == 1) {
         if (blockIdx.x >= grid_rows) return;
         const int nchunk = ceil_div(s.COg, 256);
@@ -267,14 +346,15 @@ __global__ __launch_bounds__(256) void inf_hot_kernel(const float* __restrict__ 
         const int n0 = (int)(blockIdx.x % (unsigned)nchunk) * 256 + wave * 64;
         if (n0 >= s.COg) return;  // whole waves
         const int g = (int)(r % s.G);
-        float best;
-        uint32_t code;
-        hot_walk<TRACK, true>(x + r * s.CIg, w + ((long)g * s.COg + n0) * s.CIg, s.CIg, min(64, s.COg - n0),
-                              mask_x + r * nword, nword, s.CIg, vec != 0, best, code);
+        hot_walk<P, true>(x + r * s.CIg, w + ((long)g * s.COg + n0) * s.CIg, x2off, s.CIg, min(64, s.COg - n0),
+                          mask_x + r * nword, nword, s.CIg, vec != 0, res);
         const int n = n0 + mine;
         if (n < s.COg) {
-            out[r * s.COg + n] = best;
-            if constexpr (TRACK) pos[r * s.COg + n] = (int32_t)code;
+            P::outputs(res, fv, iv);
+#pragma unroll
+            for (int c = 0; c < NF; c++) out.f[c][r * s.COg + n] = fv[c];
+#pragma unroll
+            for (int c = 0; c < NI; c++) out.i[c][r * s.COg + n] = (int32_t)iv[c];
         }
     } else if (choice == 2) {
         if (blockIdx.x >= grid_cols) return;
@@ -287,15 +367,17 @@ __global__ __launch_bounds__(256) void inf_hot_kernel(const float* __restrict__ 
         // HW == 1: row m of group g of x starts at (m * G + g) * CIg, consecutive rows are G * CIg apart
         for (int i = 0; i < 4; i++) {
             const int c = wave * 4 + i, n = nb * 16 + c;
-            float best = kEps;
-            uint32_t code = 0;
+            P::init(res);
             if (n < s.COg) {  // wave-uniform
                 const long wrow = (long)g * s.COg + n;
-                hot_walk<TRACK, false>(w + wrow * s.CIg, x + ((long)m0 * s.G + g) * s.CIg, (long)s.CIg * s.G,
-                                       min(64, s.M - m0), mask_w + wrow * nword, nword, s.CIg, vec != 0, best, code);
+                hot_walk<P, false>(w + wrow * s.CIg, x + ((long)m0 * s.G + g) * s.CIg, x2off, (long)s.CIg * s.G,
+                                   min(64, s.M - m0), mask_w + wrow * nword, nword, s.CIg, vec != 0, res);
             }
-            tv[mine][c] = best;
-            if constexpr (TRACK) tc[mine][c] = code;
+            P::outputs(res, fv, iv);
+#pragma unroll
+            for (int e = 0; e < NF; e++) tv[e][mine][c] = fv[e];
+#pragma unroll
+            for (int e = 0; e < NI; e++) tc[e][mine][c] = iv[e];
         }
         __syncthreads();
         const int mr = threadIdx.x >> 2, mo = m0 + mr, c0 = (threadIdx.x & 3) * 4;
@@ -305,8 +387,10 @@ __global__ __launch_bounds__(256) void inf_hot_kernel(const float* __restrict__ 
                 const int n = nb * 16 + c0 + j;
                 if (n < s.COg) {
                     const long o = ((long)mo * s.G + g) * s.COg + n;
-                    out[o] = tv[mr][c0 + j];
-                    if constexpr (TRACK) pos[o] = (int32_t)tc[mr][c0 + j];
+#pragma unroll
+                    for (int e = 0; e < NF; e++) out.f[e][o] = tv[e][mr][c0 + j];
+#pragma unroll
+                    for (int e = 0; e < NI; e++) out.i[e][o] = (int32_t)tc[e][mr][c0 + j];
                 }
             }
         }
@@ -335,8 +419,8 @@ size_t hot_scratch_floats(const Geom& s) {
     return 8 + 2 * (size_t)plan_blocks(s) + nword * ((size_t)s.M * s.G + (size_t)s.COg * s.G);
 }
 
-int launch_inf_hot(const float* x, const float* w, const Geom& s, const SeedBuffers& sb, float* base, float* out,
-                   int32_t* pos, hipStream_t st, const int** decision) {
+static int launch_hot(const float* x, const float* x2, const float* w, const Geom& s, const SeedBuffers& sb, float* base,
+                      const HotOut& out, bool track, hipStream_t st, const int** decision) {
     const int ntile = sb.ntile, nword = ceil_div(ntile, 32), nblk = plan_blocks(s);
     const long rows = (long)s.M * s.G;
     int* dec = reinterpret_cast<int*>(base);  // [0] decision, [1], [2] hot entries per side, [3] ticket (cleared by the row pre-pass)
@@ -346,18 +430,38 @@ int launch_inf_hot(const float* x, const float* w, const Geom& s, const SeedBuff
     *decision = dec;
     // at most 1 / 32 of all (row, column, tile) triples: beyond that the k-tile skipping dense kernel is the faster one
     hipLaunchKernelGGL(hot_plan_kernel, dim3(nblk), dim3(1024), 2 * s.G * sizeof(unsigned), st, sb.seed_x, sb.seed_w,
-                       sb.tile_x, sb.tile_w, s, ntile, nword, mask_x, mask_w, dec, partial, hot_mode(), 32);
-    const int vec = s.CIg % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0;
+                       sb.tile_x, sb.tile_w, s, ntile, nword, mask_x, mask_w, dec, partial, hot_mode(), 32,
+                       x2 != nullptr ? sb.far_hi : nullptr, x2 != nullptr ? sb.far_lo : nullptr);
+    int vec = s.CIg % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0;
+    if (x2 != nullptr) vec = vec && (uintptr_t)x2 % 16 == 0;
+    const long x2off = x2 != nullptr ? (long)(((intptr_t)x2 - (intptr_t)x) / (intptr_t)sizeof(float)) : 0;
     const unsigned grid_r = (unsigned)(rows * ceil_div(s.COg, 256));
     const unsigned grid_c = (unsigned)((long)ceil_div(s.M, 64) * ceil_div(s.COg, 16) * s.G);
     const dim3 grid(grid_r > grid_c ? grid_r : grid_c);
-    if (pos != nullptr)
-        hipLaunchKernelGGL(inf_hot_kernel<true>, grid, dim3(256), 0, st, x, w, s, mask_x, mask_w, nword, vec, out, pos, dec,
-                           grid_r, grid_c);
-    else
-        hipLaunchKernelGGL(inf_hot_kernel<false>, grid, dim3(256), 0, st, x, w, s, mask_x, mask_w, nword, vec, out, pos, dec,
-                           grid_r, grid_c);
+#define NDIST_HOT(POLICY) \
+    hipLaunchKernelGGL(hot_kernel<POLICY>, grid, dim3(256), 0, st, x, x2off, w, s, mask_x, mask_w, nword, vec, out, dec, \
+                       grid_r, grid_c)
+    if (x2 == nullptr) {
+        if (track) NDIST_HOT(HotInf<true>);
+        else NDIST_HOT(HotInf<false>);
+    } else {
+        if (track) NDIST_HOT(HotBound<true>);
+        else NDIST_HOT(HotBound<false>);
+    }
+#undef NDIST_HOT
     return hip_failed(hipGetLastError()) ? 4 : 0;
+}
+
+int launch_inf_hot(const float* x, const float* w, const Geom& s, const SeedBuffers& sb, float* base, float* out,
+                   int32_t* pos, hipStream_t st, const int** decision) {
+    const HotOut o{{out, nullptr}, {pos, nullptr}};
+    return launch_hot(x, nullptr, w, s, sb, base, o, pos != nullptr, st, decision);
+}
+
+int launch_bound_hot(const float* xl, const float* xu, const float* w, const Geom& s, const SeedBuffers& sb, float* base,
+                     float* yl, float* yu, int32_t* pl, int32_t* pu, hipStream_t st, const int** decision) {
+    const HotOut o{{yl, yu}, {pl, pu}};
+    return launch_hot(xl, xu, w, s, sb, base, o, pl != nullptr, st, decision);
 }
 
 }  // namespace ndist

@@ -436,6 +436,10 @@ struct SeedSide {
     float* seed;
     int32_t* seed_k;
     float* tile_max;
+    // interval bounds, optional: per row the largest max(-lower, upper) and the largest max(lower, -upper) over k,
+    // inverted boxes collapsed to their midpoint first (NaN when the row holds a NaN)
+    float* out_hi;
+    float* out_lo;
 };
 __device__ __forceinline__ void norm_seed_row(const SeedSide& sd, long r, int ntile) {
     const int lane = threadIdx.x & 63;
@@ -447,6 +451,7 @@ __device__ __forceinline__ void norm_seed_row(const SeedSide& sd, long r, int nt
     float best = -1.f, val = 0.f;
     int bk = 0;
     bool bad = false;  // a NaN in the row (or +inf next to -inf): the pair at the row's seed may not exist
+    float far_hi = -__builtin_inff(), far_lo = -__builtin_inff();
     if (K % 4 == 0 && (uintptr_t)x % 16 == 0 && xq == nullptr) {  // 16-byte loads: 1 KiB per wave and iteration
         for (int k0 = 0; k0 < K; k0 += 256) {
             const int k = k0 + 4 * lane;
@@ -477,6 +482,10 @@ __device__ __forceinline__ void norm_seed_row(const SeedSide& sd, long r, int nt
                 if (xq != nullptr) {
                     const float v2 = xq[k];
                     bad |= v2 != v2;
+                    float lo = v, up = v2;
+                    if (lo > up) lo = up = (lo + up) * 0.5f;
+                    far_hi = fmaxf(far_hi, fmaxf(-lo, up));
+                    far_lo = fmaxf(far_lo, fmaxf(lo, -up));
                     v = fabsf(v2) > fabsf(v) ? v2 : v;
                 }
                 local = fabsf(v);
@@ -496,6 +505,17 @@ __device__ __forceinline__ void norm_seed_row(const SeedSide& sd, long r, int nt
     // a row with a NaN is marked by a NaN seed value: consumers that form pairs with it drop them like any NaN pair
     if (__builtin_amdgcn_ballot_w64(bad) != 0) val = __builtin_nanf("");
     if (lane == 0) { sd.seed[r] = val; sd.seed_k[r] = bk; }
+    if (sd.out_hi != nullptr) {
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) {
+            far_hi = fmaxf(far_hi, __shfl_xor(far_hi, d, 64));
+            far_lo = fmaxf(far_lo, __shfl_xor(far_lo, d, 64));
+        }
+        if (lane == 0) {
+            sd.out_hi[r] = val == val ? far_hi : val;
+            sd.out_lo[r] = val == val ? far_lo : val;
+        }
+    }
 }
 
 
@@ -639,6 +659,10 @@ size_t seed_scratch_floats(const Geom& s) {
     return (2 + (size_t)ceil_div(s.CIg, 32)) * (rows + wrows) + total;
 }
 
+size_t bound_seed_scratch_floats(const Geom& s) {
+    return seed_scratch_floats(s) + (size_t)s.M * s.COg * s.G + 2 * (size_t)s.M * s.G;
+}
+
 size_t weight_seed_floats(const Geom& s) {
     return (2 + (size_t)ceil_div(s.CIg, 32)) * ((size_t)s.COg * s.G);
 }
@@ -650,7 +674,7 @@ int launch_weight_seeds(const float* w, const Geom& s, float* base, const int* g
     out->seed_w = base;
     out->seed_wk = reinterpret_cast<int32_t*>(base + wrows);
     out->tile_w = reinterpret_cast<float*>(out->seed_wk + wrows);
-    const SeedSide sw{w, nullptr, wrows, s.CIg, out->seed_w, out->seed_wk, out->tile_w};
+    const SeedSide sw{w, nullptr, wrows, s.CIg, out->seed_w, out->seed_wk, out->tile_w, nullptr, nullptr};
     hipLaunchKernelGGL(norm_seed_kernel, dim3((unsigned)((wrows + 3) / 4)), dim3(256), 0, st, sw, SeedSide{}, (int)((wrows + 3) / 4),
                        ntile, gate, gate_limit, (int*)nullptr);
     return hip_failed(hipGetLastError()) ? 4 : 0;
@@ -675,8 +699,11 @@ int launch_row_seeds(const float* x, const float* w, const Geom& s, float* base,
         tile_w = wpre->tile_w;
     }
     // one launch for the rows of x and (unless done before) the rows of w
-    const SeedSide sx{x, x2, rows, s.CIg, seed_x, seed_k, tile_x};
-    const SeedSide sw{w, nullptr, wpre != nullptr ? 0 : wrows, s.CIg, seed_w, seed_wk, tile_w};
+    // (interval bounds: the two extra row statistics lie behind the second seed array)
+    float* far_hi = x2 != nullptr ? after_tiles + total : nullptr;
+    float* far_lo = x2 != nullptr ? far_hi + rows : nullptr;
+    const SeedSide sx{x, x2, rows, s.CIg, seed_x, seed_k, tile_x, far_hi, far_lo};
+    const SeedSide sw{w, nullptr, wpre != nullptr ? 0 : wrows, s.CIg, seed_w, seed_wk, tile_w, nullptr, nullptr};
     const int nbx = (int)((rows + 3) / 4), nbw = (int)((sw.rows + 3) / 4);
     hipLaunchKernelGGL(norm_seed_kernel, dim3((unsigned)(nbx + nbw)), dim3(256), 0, st, sx, sw, nbx, ntile, gate, gate_limit,
                        zero);
@@ -686,6 +713,8 @@ int launch_row_seeds(const float* x, const float* w, const Geom& s, float* base,
     out->tile_x = tile_x;
     out->tile_w = tile_w;
     out->ntile = ntile;
+    out->far_hi = far_hi;
+    out->far_lo = far_lo;
     out->seed_x = seed_x;
     out->seed_k = seed_k;
     out->seed_w = seed_w;

@@ -119,6 +119,9 @@ struct SeedBuffers {
     int32_t* seed_k;
     float* seed_w;
     int32_t* seed_wk;
+    // interval bounds only: per row of the box the largest max(-lower, upper) and max(lower, -upper) over k
+    float* far_hi;
+    float* far_lo;
 };
 // The part of the pre-passes that depends on w alone (per row of w: largest element, its k, tile maxima): two
 // operators called on the same weights (a layer's distance and its interval bounds) can share it.
@@ -128,6 +131,7 @@ struct WeightSeeds {
     float* tile_w;
 };
 size_t seed_scratch_floats(const Geom& s);
+size_t bound_seed_scratch_floats(const Geom& s);  // with the second seed array and the row statistics of the box
 size_t weight_seed_floats(const Geom& s);
 int launch_weight_seeds(const float* w, const Geom& s, float* base, const int* gate, int gate_limit, hipStream_t st,
                         WeightSeeds* out);
@@ -153,6 +157,9 @@ bool hot_forward_applies(const Geom& s);
 size_t hot_scratch_floats(const Geom& s);
 int launch_inf_hot(const float* x, const float* w, const Geom& s, const SeedBuffers& sb, float* base, float* out,
                    int32_t* pos, hipStream_t st, const int** decision);
+// the same for the interval bounds (sb from the row pre-pass over both input bounds)
+int launch_bound_hot(const float* xl, const float* xu, const float* w, const Geom& s, const SeedBuffers& sb, float* base,
+                     float* yl, float* yu, int32_t* pl, int32_t* pu, hipStream_t st, const int** decision);
 void set_hot_mode(int mode);
 int hot_mode();
 

@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 from oracle import norm_dist_oracle as O
-from util import gpu_inf_forward
+from util import gpu_bound_forward, gpu_inf_forward
 
 pytestmark = pytest.mark.gpu
 
@@ -76,6 +76,39 @@ def test_hot_tiles_match_the_oracle(modes, B, CO, CI, G, kind, mode):
     assert np.array_equal(out2.view(np.uint32), eo.view(np.uint32)), "values without codes %s mode %d" % (kind, mode)
 
 
+def _boxes(kind, x, r):
+    """Input bounds around x: narrow boxes, boxes as wide as the data (the lower reduction then sees its floor),
+    some inverted boxes (they collapse to their midpoint), and with `special` data the NaN / infinities of x."""
+    radius = {"wide": 2.0}.get(kind, 8.0 / 255.0)
+    xl, xu = (x - radius).astype(np.float32), (x + radius).astype(np.float32)
+    flip = r.rand(*x.shape) < 0.02
+    xl[flip], xu[flip] = xu[flip].copy(), xl[flip].copy()
+    return xl, xu
+
+
+@pytest.mark.parametrize("mode", [2, 3, 1, -1, 0])
+@pytest.mark.parametrize("kind", ["small_w", "diagonal", "normal", "ties", "floor", "special", "wide"])
+@pytest.mark.parametrize("B,CO,CI,G", SHAPES)
+def test_hot_tiles_interval_bounds_match_the_oracle(modes, B, CO, CI, G, kind, mode):
+    """The same for the interval bounds (reference: core/cuda/bound_inf_dist_cuda.cu:63,148-151,203-213,225-232):
+    both bounds and both arg codes, with the "no gradient" code where the lower reduction stays at its floor."""
+    if kind == "floor" and CO % G:
+        pytest.skip("needs whole groups")
+    modes(mode)
+    x, w = _data("small_w" if kind == "wide" else kind, B, CO, CI, G, seed=B + CO + 1)
+    xl, xu = _boxes(kind, x, np.random.RandomState(B))
+    el, eu, epl, epu = O.bound_inf_dist_forward(xl, xu, w, G)
+    yl, yu, pl, pu = gpu_bound_forward(xl, xu, w, G)
+    what = "%s mode %d" % (kind, mode)
+    assert np.array_equal(yl.view(np.uint32), el.view(np.uint32)), "lower bound " + what
+    assert np.array_equal(yu.view(np.uint32), eu.view(np.uint32)), "upper bound " + what
+    assert np.array_equal(pl, epl), "codes of the lower bound " + what
+    assert np.array_equal(pu, epu), "codes of the upper bound " + what
+    yl2, yu2, _, _ = gpu_bound_forward(xl, xu, w, G, with_pos=False)
+    assert np.array_equal(yl2.view(np.uint32), el.view(np.uint32)), "lower bound without codes " + what
+    assert np.array_equal(yu2.view(np.uint32), eu.view(np.uint32)), "upper bound without codes " + what
+
+
 def test_decision_follows_the_data(modes):
     """With the counts deciding, both kinds of sparse data and dense data give the oracle's bits at a size where the
     choice matters (the kernel names in a profile tell which path ran; here only the results are checked)."""
@@ -86,3 +119,8 @@ def test_decision_follows_the_data(modes):
         eo, ep = O.inf_dist_forward(x, w)
         out, pos = gpu_inf_forward(x, w)
         assert np.array_equal(out, eo) and np.array_equal(pos, ep), kind
+        xl, xu = _boxes(kind, x, np.random.RandomState(3))
+        expect = O.bound_inf_dist_forward(xl, xu, w)
+        got = gpu_bound_forward(xl, xu, w)
+        for e, v in zip(expect, got):
+            assert np.array_equal(e, v), "interval bounds " + kind
