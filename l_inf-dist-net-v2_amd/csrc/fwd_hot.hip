@@ -243,9 +243,11 @@ struct HotBound {  // interval bounds (core/cuda/bound_inf_dist_cuda.cu:63,148-1
 // One wave: the hot tiles of one owner row (bits of mk, ascending k) against 64 rows of the other side.  Eight lanes
 // share a row of the other side and split a 32-wide tile into 16-byte pieces (a load instruction then covers eight
 // whole 128-byte rows instead of 64 different cache lines), lane group q of the wave serves the rows q, q + 8, ...,
-// q + 56 past `oth`, `stride` floats apart (`nrow` of them exist; the others re-read the first row and are
+// q + 8 * (kHotSlots - 1) past `oth`, `stride` floats apart (`nrow` of them exist; the others re-read the first row and are
 // discarded by the caller).  X_OWNS: the owner is the row of x.  x has a second array at distance `x2off` floats
 // for the interval bounds (P::NX == 2).  Every lane ends with the result of row 8 * (lane & 7) + (lane >> 3).
+constexpr int kHotSlots = 4;               // rows of the other side per lane group
+constexpr int kHotRows = 8 * kHotSlots;    // rows of the other side per wave
 template <class P, bool X_OWNS>
 __device__ __forceinline__ void hot_walk(const float* __restrict__ own, const float* __restrict__ oth, long x2off,
                                          long stride, int nrow, const uint32_t* __restrict__ mk, int nword, int K,
@@ -253,10 +255,10 @@ __device__ __forceinline__ void hot_walk(const float* __restrict__ own, const fl
     using State = typename P::State;
     constexpr bool TWO = P::NX == 2;
     const int lane = threadIdx.x & 63, sub = lane & 7, q = lane >> 3;
-    State st[8];
-    const float* rowp[8];
+    State st[kHotSlots];
+    const float* rowp[kHotSlots];
 #pragma unroll
-    for (int j = 0; j < 8; j++) {
+    for (int j = 0; j < kHotSlots; j++) {
         P::init(st[j]);
         const int row = q + 8 * j;
         rowp[j] = oth + (long)(row < nrow ? row : 0) * stride;
@@ -270,14 +272,14 @@ __device__ __forceinline__ void hot_walk(const float* __restrict__ own, const fl
                 const float4 o = *reinterpret_cast<const float4*>(own + k0);
                 float4 o2 = o;
                 if constexpr (TWO && X_OWNS) o2 = *reinterpret_cast<const float4*>(own + x2off + k0);
-                float4 v[8], v2[TWO && !X_OWNS ? 8 : 1];
+                float4 v[kHotSlots], v2[TWO && !X_OWNS ? kHotSlots : 1];
 #pragma unroll
-                for (int j = 0; j < 8; j++) {
+                for (int j = 0; j < kHotSlots; j++) {
                     v[j] = *reinterpret_cast<const float4*>(rowp[j] + k0);
                     if constexpr (TWO && !X_OWNS) v2[j] = *reinterpret_cast<const float4*>(rowp[j] + x2off + k0);
                 }
 #pragma unroll
-                for (int j = 0; j < 8; j++) {
+                for (int j = 0; j < kHotSlots; j++) {
                     if constexpr (X_OWNS) {
                         P::pair(st[j], o.x, o2.x, v[j].x, k0 + 0);
                         P::pair(st[j], o.y, o2.y, v[j].y, k0 + 1);
@@ -296,7 +298,7 @@ __device__ __forceinline__ void hot_walk(const float* __restrict__ own, const fl
                 for (int k = k0; k < k1; k++) {
                     const float o = own[k], o2 = TWO && X_OWNS ? own[x2off + k] : o;
 #pragma unroll
-                    for (int j = 0; j < 8; j++) {
+                    for (int j = 0; j < kHotSlots; j++) {
                         if constexpr (X_OWNS) P::pair(st[j], o, o2, rowp[j][k], k);
                         else P::pair(st[j], rowp[j][k], TWO ? rowp[j][x2off + k] : 0.f, o, k);
                     }
@@ -306,13 +308,13 @@ __device__ __forceinline__ void hot_walk(const float* __restrict__ own, const fl
     }
     // the eight lanes of a row merge
 #pragma unroll
-    for (int j = 0; j < 8; j++) {
+    for (int j = 0; j < kHotSlots; j++) {
 #pragma unroll
         for (int d = 1; d < 8; d <<= 1) P::merge_xor(st[j], d);
     }
     res = st[0];
 #pragma unroll
-    for (int j = 1; j < 8; j++) P::select(res, st[j], sub == j);
+    for (int j = 1; j < kHotSlots; j++) P::select(res, st[j], sub == j);
 }
 
 struct HotOut {
@@ -331,25 +333,27 @@ __global__ __launch_bounds__(256) void hot_kernel(const float* __restrict__ x, l
                                                   const uint32_t* __restrict__ mask_w, int nword, int vec, const HotOut out,
                                                   const int* __restrict__ dec, unsigned grid_rows, unsigned grid_cols) {
     constexpr int NF = P::NF, NI = P::NI;
-    __shared__ float tv[NF][64][17];
-    __shared__ uint32_t tc[NI > 0 ? NI : 1][64][17];
+    __shared__ float tv[NF][kHotRows][17];
+    __shared__ uint32_t tc[NI > 0 ? NI : 1][kHotRows][17];
     const int choice = dec[0];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int mine = 8 * (lane & 7) + (lane >> 3);  // the row of the other side whose result this lane ends up with
+    // the row of the other side whose result this lane ends up with (lanes with (lane & 7) >= kHotSlots: none)
+    const int mine = 8 * (lane & 7) + (lane >> 3);
+    const bool reports = (lane & 7) < kHotSlots;
     typename P::State res;
     float fv[NF];
     uint32_t iv[NI > 0 ? NI : 1];
     if (choice == 1) {
         if (blockIdx.x >= grid_rows) return;
-        const int nchunk = ceil_div(s.COg, 256);
+        const int nchunk = ceil_div(s.COg, 4 * kHotRows);
         const long r = blockIdx.x / (unsigned)nchunk;  // row (m, g) of x
-        const int n0 = (int)(blockIdx.x % (unsigned)nchunk) * 256 + wave * 64;
+        const int n0 = (int)(blockIdx.x % (unsigned)nchunk) * 4 * kHotRows + wave * kHotRows;
         if (n0 >= s.COg) return;  // whole waves
         const int g = (int)(r % s.G);
-        hot_walk<P, true>(x + r * s.CIg, w + ((long)g * s.COg + n0) * s.CIg, x2off, s.CIg, min(64, s.COg - n0),
+        hot_walk<P, true>(x + r * s.CIg, w + ((long)g * s.COg + n0) * s.CIg, x2off, s.CIg, min(kHotRows, s.COg - n0),
                           mask_x + r * nword, nword, s.CIg, vec != 0, res);
         const int n = n0 + mine;
-        if (n < s.COg) {
+        if (reports && n < s.COg) {
             P::outputs(res, fv, iv);
 #pragma unroll
             for (int c = 0; c < NF; c++) out.f[c][r * s.COg + n] = fv[c];
@@ -358,12 +362,12 @@ __global__ __launch_bounds__(256) void hot_kernel(const float* __restrict__ x, l
         }
     } else if (choice == 2) {
         if (blockIdx.x >= grid_cols) return;
-        const int nmb = ceil_div(s.M, 64), nnb = ceil_div(s.COg, 16);
+        const int nmb = ceil_div(s.M, kHotRows), nnb = ceil_div(s.COg, 16);
         unsigned id = blockIdx.x;
         const int mb = (int)(id % (unsigned)nmb);
         id /= (unsigned)nmb;
         const int nb = (int)(id % (unsigned)nnb), g = (int)(id / (unsigned)nnb);
-        const int m0 = mb * 64;
+        const int m0 = mb * kHotRows;
         // HW == 1: row m of group g of x starts at (m * G + g) * CIg, consecutive rows are G * CIg apart
         for (int i = 0; i < 4; i++) {
             const int c = wave * 4 + i, n = nb * 16 + c;
@@ -371,17 +375,19 @@ __global__ __launch_bounds__(256) void hot_kernel(const float* __restrict__ x, l
             if (n < s.COg) {  // wave-uniform
                 const long wrow = (long)g * s.COg + n;
                 hot_walk<P, false>(w + wrow * s.CIg, x + ((long)m0 * s.G + g) * s.CIg, x2off, (long)s.CIg * s.G,
-                                   min(64, s.M - m0), mask_w + wrow * nword, nword, s.CIg, vec != 0, res);
+                                   min(kHotRows, s.M - m0), mask_w + wrow * nword, nword, s.CIg, vec != 0, res);
             }
             P::outputs(res, fv, iv);
+            if (reports) {
 #pragma unroll
-            for (int e = 0; e < NF; e++) tv[e][mine][c] = fv[e];
+                for (int e = 0; e < NF; e++) tv[e][mine][c] = fv[e];
 #pragma unroll
-            for (int e = 0; e < NI; e++) tc[e][mine][c] = iv[e];
+                for (int e = 0; e < NI; e++) tc[e][mine][c] = iv[e];
+            }
         }
         __syncthreads();
         const int mr = threadIdx.x >> 2, mo = m0 + mr, c0 = (threadIdx.x & 3) * 4;
-        if (mo < s.M) {
+        if (mr < kHotRows && mo < s.M) {
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const int n = nb * 16 + c0 + j;
@@ -435,8 +441,8 @@ static int launch_hot(const float* x, const float* x2, const float* w, const Geo
     int vec = s.CIg % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0;
     if (x2 != nullptr) vec = vec && (uintptr_t)x2 % 16 == 0;
     const long x2off = x2 != nullptr ? (long)(((intptr_t)x2 - (intptr_t)x) / (intptr_t)sizeof(float)) : 0;
-    const unsigned grid_r = (unsigned)(rows * ceil_div(s.COg, 256));
-    const unsigned grid_c = (unsigned)((long)ceil_div(s.M, 64) * ceil_div(s.COg, 16) * s.G);
+    const unsigned grid_r = (unsigned)(rows * ceil_div(s.COg, 4 * kHotRows));
+    const unsigned grid_c = (unsigned)((long)ceil_div(s.M, kHotRows) * ceil_div(s.COg, 16) * s.G);
     const dim3 grid(grid_r > grid_c ? grid_r : grid_c);
 #define NDIST_HOT(POLICY) \
     hipLaunchKernelGGL(hot_kernel<POLICY>, grid, dim3(256), 0, st, x, x2off, w, s, mask_x, mask_w, nword, vec, out, dec, \

@@ -453,24 +453,34 @@ __device__ __forceinline__ void norm_seed_row(const SeedSide& sd, long r, int nt
     bool bad = false;  // a NaN in the row (or +inf next to -inf): the pair at the row's seed may not exist
     float far_hi = -__builtin_inff(), far_lo = -__builtin_inff();
     if (K % 4 == 0 && (uintptr_t)x % 16 == 0 && xq == nullptr) {  // 16-byte loads: 1 KiB per wave and iteration
-        for (int k0 = 0; k0 < K; k0 += 256) {
-            const int k = k0 + 4 * lane;
-            float local = 0.f;  // largest magnitude of my four k: they lie in one tile, 8 lanes share a tile
-            if (k < K) {
-                const float4 v4 = *reinterpret_cast<const float4*>(xp + k);
-                const float v[4] = {v4.x, v4.y, v4.z, v4.w};
-                const float sum4 = (v4.x + v4.y) + (v4.z + v4.w);
-                bad |= sum4 != sum4;
+        // four loads in flight per lane: a wave alone keeps 4 KiB of the row on its way
+        for (int k0 = 0; k0 < K; k0 += 1024) {
+            float4 v4[4];
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    local = fmaxf(local, fabsf(v[j]));
-                    if (fabsf(v[j]) > best) { best = fabsf(v[j]); val = v[j]; bk = k + j; }
-                }
+            for (int u = 0; u < 4; u++) {
+                const int k = k0 + 256 * u + 4 * lane;
+                v4[u] = k < K ? *reinterpret_cast<const float4*>(xp + k) : make_float4(0.f, 0.f, 0.f, 0.f);
             }
-            local = fmaxf(local, __shfl_xor(local, 1, 64));
-            local = fmaxf(local, __shfl_xor(local, 2, 64));
-            local = fmaxf(local, __shfl_xor(local, 4, 64));
-            if ((lane & 7) == 0 && k < K) tm[k >> 5] = local;
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int k = k0 + 256 * u + 4 * lane;
+                if (k0 + 256 * u >= K) break;  // wave-uniform
+                float local = 0.f;  // largest magnitude of my four k: they lie in one tile, 8 lanes share a tile
+                if (k < K) {
+                    const float v[4] = {v4[u].x, v4[u].y, v4[u].z, v4[u].w};
+                    const float sum4 = (v[0] + v[1]) + (v[2] + v[3]);
+                    bad |= sum4 != sum4;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        local = fmaxf(local, fabsf(v[j]));
+                        if (fabsf(v[j]) > best) { best = fabsf(v[j]); val = v[j]; bk = k + j; }
+                    }
+                }
+                local = fmaxf(local, __shfl_xor(local, 1, 64));
+                local = fmaxf(local, __shfl_xor(local, 2, 64));
+                local = fmaxf(local, __shfl_xor(local, 4, 64));
+                if ((lane & 7) == 0 && k < K) tm[k >> 5] = local;
+            }
         }
     } else {
         for (int k0 = 0; k0 < K; k0 += 64) {
