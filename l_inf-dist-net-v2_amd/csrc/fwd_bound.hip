@@ -183,19 +183,19 @@ int launch_bound_forward(const float* xl, const float* xu, const float* w, const
     P.s = s;
     // large fully-connected problems: hot-tile kernels first, else seeds and k-tile bounds, as in launch_inf_forward
     const bool bounded = cv == nullptr && seeded_forward_applies(s);
-    if (!bounded && pl == nullptr) return launch_fwd_conv<OpBound<false>, CfgBoundN, CfgMid, CfgSmall>(P, st);
-    const bool hot = bounded && hot_forward_applies(s);
+    const bool hot = cv == nullptr && hot_forward_applies(s) && (bounded || hot_alone_applies(s));
+    if (!bounded && !hot && pl == nullptr) return launch_fwd_conv<OpBound<false>, CfgBoundN, CfgMid, CfgSmall>(P, st);
     KernelTimer timer(st);  // pre-passes + tiled kernel + rescan
     float* scratch = nullptr;
     const int* gate = nullptr;
-    if (bounded) {
+    if (bounded || hot) {
         const size_t nseed = bound_seed_scratch_floats(s);
         NDIST_HIP_TRY(scratch_alloc((void**)&scratch, (nseed + (hot ? hot_scratch_floats(s) : 0)) * sizeof(float), st));
         SeedBuffers sb{};
         int rs = launch_row_seeds(xl, w, s, scratch, nullptr, 0, st, &sb, xu, wpre,
                                   hot ? reinterpret_cast<int*>(scratch + nseed) : nullptr);
         if (!rs && hot) rs = launch_bound_hot(xl, xu, w, s, sb, scratch + nseed, yl, yu, pl, pu, st, &gate);
-        if (!rs) rs = launch_output_seeds(xl, w, s, sb, gate, 1, st, xu);
+        if (!rs && bounded) rs = launch_output_seeds(xl, w, s, sb, gate, 1, st, xu);
         if (rs) {
             (void)scratch_free(scratch, st);
             return rs;
@@ -205,18 +205,23 @@ int launch_bound_forward(const float* xl, const float* xu, const float* w, const
             P.gate_limit = 1;
             P.gate_sense = 1;
         }
-        P.aux = sb.seed;
-        P.aux2 = sb.seed2;
-        P.tile_x = sb.tile_x;
-        P.tile_w = sb.tile_w;
-        P.ntile32 = sb.ntile;
+        if (bounded) {
+            P.aux = sb.seed;
+            P.aux2 = sb.seed2;
+            P.tile_x = sb.tile_x;
+            P.tile_w = sb.tile_w;
+            P.ntile32 = sb.ntile;
+        }
     }
     // (the scratch holds the gate: it is released after the last kernel that reads it has been queued)
     auto done = [&](int rc) {
-        if (bounded && hip_failed(scratch_free(scratch, st)) && !rc) rc = 4;
+        if ((bounded || hot) && hip_failed(scratch_free(scratch, st)) && !rc) rc = 4;
         return rc;
     };
-    if (pl == nullptr) return done(launch_fwd<OpBound<false, true>, CfgBoundT, CfgMid, CfgSmall>(P, st));
+    if (pl == nullptr) {
+        return done(bounded ? launch_fwd<OpBound<false, true>, CfgBoundT, CfgMid, CfgSmall>(P, st)
+                            : launch_fwd_conv<OpBound<false>, CfgBoundN, CfgMid, CfgSmall>(P, st));
+    }
     int kt = 0;
     const int rc = bounded ? launch_fwd_layouts<false, OpBound<true, true>, CfgBoundT, CfgSmall>(P, st, &kt)
                            : launch_fwd_layouts<true, OpBound<true>, CfgBoundT, CfgSmall>(P, st, &kt);
@@ -245,7 +250,7 @@ int launch_bound_forward(const float* xl, const float* xu, const float* w, const
 // pre-pass over w (the largest of the pre-passes: it reads all of w) runs once and serves both operators.
 int launch_inf_bound_forward(const float* x, const float* xl, const float* xu, const float* w, const Geom& s, float* out,
                              int32_t* pos, float* yl, float* yu, int32_t* pl, int32_t* pu, hipStream_t st) {
-    if (!seeded_forward_applies(s)) {
+    if (!seeded_forward_applies(s) && !(hot_forward_applies(s) && hot_alone_applies(s))) {
         const int rc = launch_inf_forward(x, w, s, out, pos, st);
         return rc ? rc : launch_bound_forward(xl, xu, w, s, yl, yu, pl, pu, st);
     }

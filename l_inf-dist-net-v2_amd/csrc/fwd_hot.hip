@@ -74,13 +74,13 @@ __device__ __forceinline__ void hot_group_maxima(const float* __restrict__ seed_
 }
 
 // One kernel for the whole plan.  Every workgroup (1024 threads) first finds MX and MW of all groups, then its 16
-// waves turn one row each (rows of x first, then rows of w) into hot-tile masks: bit t of a row's mask = tile t is
-// hot.  The workgroups leave their counts of hot (row, tile) entries per side in `partial`; the last one to finish
-// (a ticket in dec[3], cleared by the row pre-pass) adds them up and decides:
+// waves turn four rows each (rows of x first, then rows of w; their loads issued together) into hot-tile masks: bit
+// t of a row's mask = tile t is hot.  The workgroups leave their counts of hot (row, tile) entries per side in
+// `partial`; the last one to finish (a ticket in dec[3], cleared by the row pre-pass) adds them up and decides:
 //   dec[0] = 1: the rows of x select the tiles, 2: the rows of w, 0: too many hot tiles, the dense kernels run.
 // Cost of a side = its hot entries x the length of the other side.  mode: 1 always the cheaper side, 2 / 3 always
 // the x / w side, else the cheaper side if it touches at most 1 / frac of all (row, column, tile) triples.
-constexpr int kPlanRows = 16;  // one row per wave: the chain of dependent loads per wave stays short
+constexpr int kPlanRows = 64, kPlanRowsPerWave = kPlanRows / 16;
 __global__ __launch_bounds__(1024) void hot_plan_kernel(const float* __restrict__ seed_x, const float* __restrict__ seed_w,
                                                         const float* __restrict__ tile_x, const float* __restrict__ tile_w,
                                                         const Geom s, int ntile, int nword, uint32_t* __restrict__ mask_x,
@@ -96,35 +96,55 @@ __global__ __launch_bounds__(1024) void hot_plan_kernel(const float* __restrict_
     hot_group_maxima(seed_x, seed_w, s, sm);
     const long rows = (long)s.M * s.G, wrows = (long)s.COg * s.G;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int i = 0; i < kPlanRows / 16; i++) {
-        const long r = (long)blockIdx.x * kPlanRows + wave * (kPlanRows / 16) + i;
-        if (r >= rows + wrows) break;  // wave-uniform
-        const bool isw = r >= rows;
-        const long rr = isw ? r - rows : r;
-        const int g = isw ? (int)(rr / s.COg) : (int)(rr % s.G);
-        const float own = fabsf(isw ? seed_w[rr] : seed_x[rr]);
-        const float other = __uint_as_float(sm[isw ? g : s.G + g]);
-        double thr = hot_threshold(own, other);
-        if (!isw && far_hi != nullptr) {
+    constexpr int R = kPlanRowsPerWave;
+    const float* tm[R];
+    uint32_t* mk[R];
+    double thr[R];
+    bool valid[R], isw[R];
+    long rr[R];
+    int count[R];
+#pragma unroll
+    for (int i = 0; i < R; i++) {
+        const long r = (long)blockIdx.x * kPlanRows + wave * R + i;
+        valid[i] = r < rows + wrows;  // wave-uniform
+        isw[i] = r >= rows;
+        rr[i] = !valid[i] ? 0 : (isw[i] ? r - rows : r);
+        const int g = isw[i] ? (int)(rr[i] / s.COg) : (int)(rr[i] % s.G);
+        const float own = fabsf(isw[i] ? seed_w[valid[i] ? rr[i] : 0] : seed_x[rr[i]]);
+        const float other = __uint_as_float(sm[isw[i] ? g : s.G + g]);
+        thr[i] = hot_threshold(own, other);
+        if (!isw[i] && far_hi != nullptr) {
             // interval bounds, rows of the box: the two reductions have their own lower bounds, far_hi - RW for the
             // upper one and far_lo - RW for the lower one; a tile is dead when it is dead for both
-            const double tu = hot_threshold(far_hi[rr], other), tl = hot_threshold(far_lo[rr], other);
-            thr = own == own ? (tu < tl ? tu : tl) : -__builtin_inf();
+            const double tu = hot_threshold(far_hi[rr[i]], other), tl = hot_threshold(far_lo[rr[i]], other);
+            thr[i] = own == own ? (tu < tl ? tu : tl) : -__builtin_inf();
         }
-        const float* __restrict__ tm = (isw ? tile_w : tile_x) + rr * ntile;
-        uint32_t* __restrict__ mk = (isw ? mask_w : mask_x) + rr * nword;
-        int count = 0;
-        for (int t0 = 0; t0 < nword * 32; t0 += 64) {
-            const int t = t0 + lane;
-            const bool hot = t < ntile && !((double)tm[t] < thr);
+        tm[i] = (isw[i] ? tile_w : tile_x) + rr[i] * ntile;
+        mk[i] = (isw[i] ? mask_w : mask_x) + rr[i] * nword;
+        count[i] = 0;
+    }
+    for (int t0 = 0; t0 < nword * 32; t0 += 64) {
+        const int t = t0 + lane;
+        float v[R];
+#pragma unroll
+        for (int i = 0; i < R; i++) v[i] = valid[i] && t < ntile ? tm[i][t] : 0.f;
+#pragma unroll
+        for (int i = 0; i < R; i++) {
+            const bool hot = valid[i] && t < ntile && !((double)v[i] < thr[i]);
             const unsigned long long bits = __builtin_amdgcn_ballot_w64(hot);
-            count += __popcll(bits);
-            if (lane == 0) {
-                mk[t0 >> 5] = (uint32_t)bits;
-                if ((t0 >> 5) + 1 < nword) mk[(t0 >> 5) + 1] = (uint32_t)(bits >> 32);
+            count[i] += __popcll(bits);
+            if (lane == 0 && valid[i]) {
+                mk[i][t0 >> 5] = (uint32_t)bits;
+                if ((t0 >> 5) + 1 < nword) mk[i][(t0 >> 5) + 1] = (uint32_t)(bits >> 32);
             }
         }
-        if (lane == 0 && count != 0) atomicAdd(&cnt[isw ? 1 : 0], count);
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int i = 0; i < R; i++) {
+            if (!valid[i]) continue;
+            if (count[i] != 0) atomicAdd(&cnt[isw[i] ? 1 : 0], count[i]);
+        }
     }
     __syncthreads();
     if (threadIdx.x == 0) {

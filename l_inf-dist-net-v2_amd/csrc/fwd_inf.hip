@@ -140,6 +140,13 @@ __global__ __launch_bounds__(256) void inf_rescan_kernel(const float* __restrict
     pos[o] = (int32_t)code;
 }
 
+// Problems below the size of the seeded kernels on which the hot-tile path is still tried first (its pre-pass reads
+// all of x and w once, so it pays from about this many pairs on); the plain kernels stay queued behind it, gated.
+bool hot_alone_applies(const Geom& s) {
+    const double pairs = (double)s.M * s.COg * s.G * s.CIg;
+    return s.HW == 1 && !skinny_applies(s) && skip_override_limit(1) > 0 && pairs >= 5e7 && s.M >= 8;
+}
+
 bool seeded_forward_applies(const Geom& s) {
     const double pairs = (double)s.M * s.COg * s.G * s.CIg;
     return s.HW == 1 && !skinny_applies(s) && skip_override_limit(1) > 0 &&
@@ -167,18 +174,18 @@ int launch_inf_forward(const float* x, const float* w, const Geom& s, float* out
     // Before those: from the same row pre-pass the hot-tile kernels (fwd_hot.hip) find out on the device whether
     // few k-tiles decide all maxima; if so they produce the outputs themselves and everything queued below is gated off.
     const bool bounded = cv == nullptr && seeded_forward_applies(s);
-    const bool hot = bounded && hot_forward_applies(s);
+    const bool hot = cv == nullptr && hot_forward_applies(s) && (bounded || hot_alone_applies(s));
     float* scratch = nullptr;
     const int* gate = nullptr;
     KernelTimer timer(st);  // pre-passes + tiled kernel + rescan
-    if (bounded) {
+    if (bounded || hot) {
         const size_t nseed = seed_scratch_floats(s);
         NDIST_HIP_TRY(scratch_alloc((void**)&scratch, (nseed + (hot ? hot_scratch_floats(s) : 0)) * sizeof(float), st));
         SeedBuffers sb{};
         int rs = launch_row_seeds(x, w, s, scratch, nullptr, 0, st, &sb, nullptr, wpre,
                                   hot ? reinterpret_cast<int*>(scratch + nseed) : nullptr);
         if (!rs && hot) rs = launch_inf_hot(x, w, s, sb, scratch + nseed, out, pos, st, &gate);
-        if (!rs) rs = launch_output_seeds(x, w, s, sb, gate, 1, st);
+        if (!rs && bounded) rs = launch_output_seeds(x, w, s, sb, gate, 1, st);
         if (rs) {
             (void)scratch_free(scratch, st);
             return rs;
@@ -188,14 +195,16 @@ int launch_inf_forward(const float* x, const float* w, const Geom& s, float* out
             P.gate_limit = 1;
             P.gate_sense = 1;
         }
-        P.aux = sb.seed;
-        P.tile_x = sb.tile_x;
-        P.tile_w = sb.tile_w;
-        P.ntile32 = sb.ntile;
+        if (bounded) {
+            P.aux = sb.seed;
+            P.tile_x = sb.tile_x;
+            P.tile_w = sb.tile_w;
+            P.ntile32 = sb.ntile;
+        }
     }
     // (the scratch holds the gate: it is released after the last kernel that reads it has been queued)
     auto done = [&](int rc) {
-        if (bounded && hip_failed(scratch_free(scratch, st)) && !rc) rc = 4;
+        if ((bounded || hot) && hip_failed(scratch_free(scratch, st)) && !rc) rc = 4;
         return rc;
     };
     if (pos == nullptr) {

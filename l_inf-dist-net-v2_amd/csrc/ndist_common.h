@@ -154,6 +154,7 @@ int launch_output_seeds(const float* x, const float* w, const Geom& s, const See
 // rows of x / of w.
 // `base` starts with the four ints the row pre-pass has to clear (launch_row_seeds' `zero`).
 bool hot_forward_applies(const Geom& s);
+bool hot_alone_applies(const Geom& s);  // fwd_inf.hip: below the size of the seeded kernels, still worth the pre-pass
 size_t hot_scratch_floats(const Geom& s);
 int launch_inf_hot(const float* x, const float* w, const Geom& s, const SeedBuffers& sb, float* base, float* out,
                    int32_t* pos, hipStream_t st, const int** decision);

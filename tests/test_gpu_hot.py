@@ -109,6 +109,31 @@ def test_hot_tiles_interval_bounds_match_the_oracle(modes, B, CO, CI, G, kind, m
     assert np.array_equal(yu2.view(np.uint32), eu.view(np.uint32)), "upper bound without codes " + what
 
 
+@pytest.mark.parametrize("mode", [-1, 2, 3])
+@pytest.mark.parametrize("kind", ["small_w", "diagonal", "normal"])
+@pytest.mark.parametrize("B,CO,CI", [(64, 1024, 1024), (8, 2560, 2560), (150, 800, 1000)])
+def test_small_batches_unforced(B, CO, CI, kind, mode):
+    """Batches below the size of the k-tile skipping kernels still try the hot tiles first (from 5e7 pairs on), with
+    the plain kernels queued behind the decision: no forcing of the seeded paths here."""
+    from core import _C
+    _C.set_hot_mode(mode)
+    try:
+        x, w = _data(kind, B, CO, CI, 1, seed=B)
+        eo, ep = O.inf_dist_forward(x, w)
+        out, pos = gpu_inf_forward(x, w)
+        assert np.array_equal(out, eo) and np.array_equal(pos, ep), "%s mode %d" % (kind, mode)
+        out2, _ = gpu_inf_forward(x, w, with_pos=False)
+        assert np.array_equal(out2, eo), "without codes %s mode %d" % (kind, mode)
+        xl, xu = _boxes(kind, x, np.random.RandomState(4))
+        expect = O.bound_inf_dist_forward(xl, xu, w)
+        for with_pos in (True, False):
+            got = gpu_bound_forward(xl, xu, w, with_pos=with_pos)
+            for e, v in zip(expect, got):
+                assert v is None or np.array_equal(e, v), "interval bounds %s mode %d" % (kind, mode)
+    finally:
+        _C.set_hot_mode(-1)
+
+
 def test_decision_follows_the_data(modes):
     """With the counts deciding, both kinds of sparse data and dense data give the oracle's bits at a size where the
     choice matters (the kernel names in a profile tell which path ran; here only the results are checked)."""
