@@ -338,9 +338,10 @@ def main():
             d["frac_issue_model"] = round(PAIRS / 64 * ISSUE_CYCLES[k] / SIMD_HZ * 1e3 / ms, 4)
             d["frac_microbench_floor"] = round(PAIRS / 64 * MICROBENCH_CYCLES[k] / SIMD_HZ * 1e3 / ms, 4)
             if k == "inf_fwd":
-                # the p = inf forward skips k-tiles that cannot matter: its rates are algorithmic (all pairs counted
-                # over the time of pre-passes + tiled kernel + second pass), not a measure of instruction issue
-                d["note"] = "k-tile skipping: algorithmic rates"
+                # the p = inf forward looks only at the k-tiles that can hold a maximum (on this data: one or two of
+                # 160 per row of x): its rates are algorithmic (all pairs counted over the time of pre-pass + plan
+                # + hot-tile kernel), not a measure of instruction issue
+                d["note"] = "hot k-tiles only: algorithmic rates"
         else:
             nbytes = 4 * (2 * B * CO + B * CI + CO * CI)  # grad_out + pos read, grad_x + grad_w written
             d["gbs"] = round(nbytes / ms / 1e6, 1)
