@@ -507,13 +507,14 @@ __global__ __launch_bounds__(64 * NW, 4) void bwd_fused_kernel(const float* __re
     flush_gx();
 }
 
-// Small batches (at most 64 rows).  The row-split kernel above would pad the rows to a whole workgroup and spend
+// Small batches (at most 32 rows; 33 to 64 rows take the two-wave configuration of the kernel above, which is a
+// third faster there: no second row chunk adding into grad_weight).  The row-split kernel above would pad the rows to a whole workgroup and spend
 // its time on the padding.  Here a workgroup owns 32 rows x one ci slab and its 16 waves split the co range
 // instead: every wave keeps the same x rows, walks over its own co, and writes its grad_weight values straight from
 // registers (complete for this row chunk).  The grad_x partials of the 16 waves are summed through LDS at the end and
 // leave with one global atomic add per element and workgroup (adding them wave by wave would pile a hundred
 // same-address atomics on every element).  The work is bound by streaming w and grad_w.
-constexpr int kBwdSmallRows = 32, kBwdSmallWaves = 16, kBwdSmallMaxM = 64;
+constexpr int kBwdSmallRows = 32, kBwdSmallWaves = 16, kBwdSmallMaxM = 32;
 
 template <int IP, bool WITH_W>
 __global__ __launch_bounds__(64 * kBwdSmallWaves) void bwd_small_kernel(const float* __restrict__ X,
@@ -622,11 +623,12 @@ struct BwdPtrs {
     float* gw;  // nullptr: input gradient only
 };
 
-// rows per wave x waves per workgroup: 512 rows (one chunk at batch 512), 256 rows, 128 rows.  Always 32 rows per
+// rows per wave x waves per workgroup: 512 rows (one chunk at batch 512), 256 rows, 128 rows, and 64 rows for batches
+// of 33 to 64 (six of those workgroups per compute unit).  Always 32 rows per
 // wave (16 cost 26 % to 92 % more per row); two or four of the smaller workgroups share a compute unit, which the
 // second launch bound (at least four waves per SIMD, i.e. at most 128 registers) makes possible.
-constexpr int kBwdCfgRows[3] = {32, 32, 32};
-constexpr int kBwdCfgWaves[3] = {16, 8, 4};
+constexpr int kBwdCfgRows[5] = {32, 32, 32, 0, 32};   // (index 3 is the small-batch kernel)
+constexpr int kBwdCfgWaves[5] = {16, 8, 4, 0, 2};
 
 // one explicit instantiation per exponent, spread over several translation units to compile in parallel
 template <int IP>
@@ -662,11 +664,13 @@ int launch_bwd_ip_impl(const BwdPtrs& a, const BwdParams& P, int cfg, int grid, 
     if (a.gw != nullptr) {
         if (cfg == 0) NDIST_BWD_LAUNCH(true, 0);
         else if (cfg == 1) NDIST_BWD_LAUNCH(true, 1);
-        else NDIST_BWD_LAUNCH(true, 2);
+        else if (cfg == 2) NDIST_BWD_LAUNCH(true, 2);
+        else NDIST_BWD_LAUNCH(true, 4);
     } else {
         if (cfg == 0) NDIST_BWD_LAUNCH(false, 0);
         else if (cfg == 1) NDIST_BWD_LAUNCH(false, 1);
-        else NDIST_BWD_LAUNCH(false, 2);
+        else if (cfg == 2) NDIST_BWD_LAUNCH(false, 2);
+        else NDIST_BWD_LAUNCH(false, 4);
     }
 #undef NDIST_BWD_LAUNCH
     return hip_failed(hipGetLastError()) ? 4 : 0;
