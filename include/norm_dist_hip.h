@@ -263,6 +263,25 @@ int ndist_conv_bound_inf_dist_backward_input_weight(const float* grad_outputL, c
                                                     int stride_w, float* grad_inputL, float* grad_inputU,
                                                     float* grad_weight, ndist_stream_t stream);
 
+/* The finite-p distance on images, same conventions: norm_dist on the patches of `input` (what the reference's
+ * NormDistConv computes through torch.nn.functional.unfold + norm_dist::forward / backward_input[_weight],
+ * core/modules/norm_dist.py:93-102, core/cuda/norm_dist.h:4-17), without the unfolded tensor: the forward extracts
+ * the patches while it loads its tiles; the backward writes them once in the row layout its kernel reads and folds
+ * the gradient rows back into the image (scratch: 8 * B * C*kh*kw * OH*OW bytes from the stream's arena).
+ *   output, grad_output  [B, CO, OH * OW]    grad_input  [B, C, H, W]    grad_weight  [CO, C/G * kh * kw] */
+int ndist_conv_norm_dist_forward(const float* input, const float* weight, int B, int C, int H, int W, int CO, int G,
+                                 int kernel_h, int kernel_w, int dilation_h, int dilation_w, int padding_h, int padding_w,
+                                 int stride_h, int stride_w, float* output, float p, ndist_stream_t stream);
+int ndist_conv_norm_dist_backward_input(const float* grad_output, const float* input, const float* weight,
+                                        const float* output, int B, int C, int H, int W, int CO, int G, int kernel_h,
+                                        int kernel_w, int dilation_h, int dilation_w, int padding_h, int padding_w,
+                                        int stride_h, int stride_w, float* grad_input, float p, ndist_stream_t stream);
+int ndist_conv_norm_dist_backward_input_weight(const float* grad_output, const float* input, const float* weight,
+                                               const float* output, int B, int C, int H, int W, int CO, int G,
+                                               int kernel_h, int kernel_w, int dilation_h, int dilation_w, int padding_h,
+                                               int padding_w, int stride_h, int stride_w, float* grad_input,
+                                               float* grad_weight, float p, ndist_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

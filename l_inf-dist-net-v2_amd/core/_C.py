@@ -93,6 +93,9 @@ _conv_inf_ng = _sig("ndist_conv_inf_dist_forward_nograd", _P, _P, *([_I] * 14), 
 _conv_bnd_ng = _sig("ndist_conv_bound_inf_dist_forward_nograd", _P, _P, _P, *([_I] * 14), _P, _P, _P)
 _conv_inf_fwd = _sig("ndist_conv_inf_dist_forward", _P, _P, *([_I] * 14), _P, _P, _P)
 _conv_bnd_fwd = _sig("ndist_conv_bound_inf_dist_forward", _P, _P, _P, *([_I] * 14), _P, _P, _P, _P, _P)
+_conv_norm_fwd = _sig("ndist_conv_norm_dist_forward", _P, _P, *([_I] * 14), _P, _F, _P)
+_conv_norm_bwd_x = _sig("ndist_conv_norm_dist_backward_input", _P, _P, _P, _P, *([_I] * 14), _P, _F, _P)
+_conv_norm_bwd_xw = _sig("ndist_conv_norm_dist_backward_input_weight", _P, _P, _P, _P, *([_I] * 14), _P, _P, _F, _P)
 _conv_inf_bwd_x = _sig("ndist_conv_inf_dist_backward_input", _P, _P, *([_I] * 14), _P, _P)
 _conv_inf_bwd_xw = _sig("ndist_conv_inf_dist_backward_input_weight", _P, _P, *([_I] * 14), _P, _P, _P)
 _conv_bnd_bwd_x = _sig("ndist_conv_bound_inf_dist_backward_input", _P, _P, _P, _P, *([_I] * 14), _P, _P, _P)
@@ -463,6 +466,42 @@ def conv_bound_inf_dist_forward_nograd(inputL, inputU, weight, outputL, outputU,
         return _ext_call(_ext.conv_bound_inf_dist_forward_nograd, inputL, inputU, weight, outputL, outputU, G,
                          list(args[6:14]))
     _run(_conv_bnd_ng, dev, _p(inputL), _p(inputU), _p(weight), *args, _p(outputL), _p(outputU))
+
+
+def conv_norm_dist_forward(input, weight, output, G, p, kernel_size, dilation, padding, stride):
+    """unfold + norm_dist_forward in one kernel for finite p: input [B, C, H, W] -> output [B, CO, OH*OW]."""
+    dev = _check({}, input=input, weight=weight, output=output)
+    args = _conv_args(input, weight, output, G, kernel_size, dilation, padding, stride)
+    if _ext is not None:
+        return _ext_call(_ext.conv_norm_dist_forward, input, weight, output, G, float(p), list(args[6:14]))
+    _run(_conv_norm_fwd, dev, _p(input), _p(weight), *args, _p(output), float(p))
+
+
+def conv_norm_dist_backward_input(grad_output, input, weight, output, grad_input, G, p, kernel_size, dilation, padding,
+                                  stride):
+    """Finite-p backward on images: grad_input [B, C, H, W] (the adjoint of the patch extraction applied)."""
+    dev = _check({}, grad_output=grad_output, input=input, weight=weight, output=output, grad_input=grad_input)
+    args = _conv_args(input, weight, output, G, kernel_size, dilation, padding, stride)
+    if grad_output.shape != output.shape or grad_input.shape != input.shape:
+        raise RuntimeError("gradients must have the shapes of output and input")
+    if _ext is not None:
+        return _ext_call(_ext.conv_norm_dist_backward_input, grad_output, input, weight, output, grad_input, G, float(p),
+                         list(args[6:14]))
+    _run(_conv_norm_bwd_x, dev, _p(grad_output), _p(input), _p(weight), _p(output), *args, _p(grad_input), float(p))
+
+
+def conv_norm_dist_backward_input_weight(grad_output, input, weight, output, grad_input, grad_weight, G, p, kernel_size,
+                                         dilation, padding, stride):
+    dev = _check({}, grad_output=grad_output, input=input, weight=weight, output=output, grad_input=grad_input,
+                 grad_weight=grad_weight)
+    args = _conv_args(input, weight, output, G, kernel_size, dilation, padding, stride)
+    if grad_output.shape != output.shape or grad_input.shape != input.shape or grad_weight.shape != weight.shape:
+        raise RuntimeError("gradients must have the shapes of output, input and weight")
+    if _ext is not None:
+        return _ext_call(_ext.conv_norm_dist_backward_input_weight, grad_output, input, weight, output, grad_input,
+                         grad_weight, G, float(p), list(args[6:14]))
+    _run(_conv_norm_bwd_xw, dev, _p(grad_output), _p(input), _p(weight), _p(output), *args, _p(grad_input),
+         _p(grad_weight), float(p))
 
 
 def conv_inf_dist_forward(input, weight, output, pos, G, kernel_size, dilation, padding, stride):

@@ -166,6 +166,36 @@ class ConvInfDistF(torch.autograd.Function):
         return (grad_x if want_x else None), grad_w, None, None, None
 
 
+class ConvNormDistF(torch.autograd.Function):
+    """Finite-p distance of a convolutional layer on images [B, C, H, W]: NormDistF on the unfolded input without the
+    unfolded tensor: the forward extracts the patches while loading its tiles and keeps the image (not its nine
+    times larger patches) for the backward, which writes the patches once in the layout its kernel reads."""
+
+    @staticmethod
+    def forward(ctx, x, weight, group, p, geometry, tag):
+        ctx.group, ctx.p, ctx.geometry, ctx.tag = group, p, geometry, tag
+        _, (oh, ow) = _C.unfold_geometry(x.shape, *geometry)
+        out = torch.empty(x.size(0), weight.size(0), oh * ow, device=x.device, dtype=torch.float32)
+        _C.conv_norm_dist_forward(x, weight, out, group, p, *geometry)
+        ctx.save_for_backward(x, weight, out)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        want_x, want_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        x, weight, out = ctx.saved_tensors
+        grad_output = grad_output.contiguous()
+        grad_x = grad_w = None
+        if want_w:
+            grad_x, grad_w = torch.empty_like(x), torch.empty_like(weight)
+            _C.conv_norm_dist_backward_input_weight(grad_output, x, weight, out, grad_x, grad_w, ctx.group, ctx.p,
+                                                    *ctx.geometry)
+        elif want_x:
+            grad_x = torch.empty_like(x)
+            _C.conv_norm_dist_backward_input(grad_output, x, weight, out, grad_x, ctx.group, ctx.p, *ctx.geometry)
+        return (grad_x if want_x else None), grad_w, None, None, None, None
+
+
 class ConvBoundInfDistF(torch.autograd.Function):
     """Interval bounds of a convolutional layer on image boxes: BoundInfDistF on the unfolded bounds, fused like
     ConvInfDistF."""
@@ -215,8 +245,19 @@ def conv_norm_dist(input, weight, p, kernel_size, dilation=1, padding=0, stride=
     """norm_dist(unfold(input), weight, p, groups) for images [B, C, H, W] (what the reference's NormDistConv
     computes, core/modules/norm_dist.py:93-102).  At p = inf the kernels extract the patches while they load their
     tiles and scatter the gradient straight into the image: neither the unfolded tensor nor its gradient is ever
-    written; values and arg-max codes are bit-identical.  Finite p unfolds (its backward reads the unfolded input)."""
+    written; values and arg-max codes are bit-identical.  Finite p works on the image too: the forward extracts the
+    patches on the fly, the backward writes them once as rows for its kernel and folds the gradient rows back."""
     need_grad = torch.is_grad_enabled() and (input.requires_grad or weight.requires_grad)
+    if not math.isinf(p) and _fused_conv_ok(input) and weight.is_cuda:
+        if p <= 0:
+            raise ValueError("p must be positive")
+        geometry = (kernel_size, dilation, padding, stride)
+        if need_grad:
+            return ConvNormDistF.apply(input.contiguous(), weight.contiguous(), groups, float(p), geometry, tag)
+        _, (oh, ow) = _C.unfold_geometry(input.shape, *geometry)
+        out = torch.empty(input.size(0), weight.size(0), oh * ow, device=input.device, dtype=torch.float32)
+        _C.conv_norm_dist_forward(input.contiguous(), weight.contiguous(), out, groups, float(p), *geometry)
+        return out
     if math.isinf(p) and _fused_conv_ok(input):
         geometry = (kernel_size, dilation, padding, stride)
         if need_grad:

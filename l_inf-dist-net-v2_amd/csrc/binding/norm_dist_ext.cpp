@@ -295,6 +295,44 @@ void conv_inf_dist_forward(const Tensor& input, const Tensor& weight, Tensor& ou
                                          IM(pos), L.stream), "conv_inf_dist_forward");
 }
 
+void conv_norm_dist_forward(const Tensor& input, const Tensor& weight, Tensor& output, int G, double p, const Geo& geo) {
+    need_geo(geo); need4d(input, "input");
+    const int dev = check_all({{"input", input, false}, {"weight", weight, false}, {"output", output, false}});
+    Launch L(dev);
+    raise_on(ndist_conv_norm_dist_forward(F(input), F(weight), IMG4(input), (int)weight.size(0), G, GEO8(geo), FM(output),
+                                          (float)p, L.stream), "conv_norm_dist_forward");
+}
+
+void conv_norm_dist_backward_input(const Tensor& grad_output, const Tensor& input, const Tensor& weight,
+                                   const Tensor& output, Tensor& grad_input, int G, double p, const Geo& geo) {
+    need_geo(geo); need4d(input, "input");
+    const int dev = check_all({{"grad_output", grad_output, false}, {"input", input, false}, {"weight", weight, false},
+                               {"output", output, false}, {"grad_input", grad_input, false}});
+    TORCH_CHECK(grad_output.sizes() == output.sizes() && grad_input.sizes() == input.sizes(),
+                "gradients must have the shapes of output and input");
+    Launch L(dev);
+    raise_on(ndist_conv_norm_dist_backward_input(F(grad_output), F(input), F(weight), F(output), IMG4(input),
+                                                 (int)weight.size(0), G, GEO8(geo), FM(grad_input), (float)p, L.stream),
+             "conv_norm_dist_backward_input");
+}
+
+void conv_norm_dist_backward_input_weight(const Tensor& grad_output, const Tensor& input, const Tensor& weight,
+                                          const Tensor& output, Tensor& grad_input, Tensor& grad_weight, int G, double p,
+                                          const Geo& geo) {
+    need_geo(geo); need4d(input, "input");
+    const int dev = check_all({{"grad_output", grad_output, false}, {"input", input, false}, {"weight", weight, false},
+                               {"output", output, false}, {"grad_input", grad_input, false},
+                               {"grad_weight", grad_weight, false}});
+    TORCH_CHECK(grad_output.sizes() == output.sizes() && grad_input.sizes() == input.sizes() &&
+                    grad_weight.sizes() == weight.sizes(),
+                "gradients must have the shapes of output, input and weight");
+    Launch L(dev);
+    raise_on(ndist_conv_norm_dist_backward_input_weight(F(grad_output), F(input), F(weight), F(output), IMG4(input),
+                                                        (int)weight.size(0), G, GEO8(geo), FM(grad_input),
+                                                        FM(grad_weight), (float)p, L.stream),
+             "conv_norm_dist_backward_input_weight");
+}
+
 void conv_bound_inf_dist_forward(const Tensor& inputL, const Tensor& inputU, const Tensor& weight, Tensor& outputL,
                                  Tensor& outputU, Tensor& posL, Tensor& posU, int G, const Geo& geo) {
     need_geo(geo); need4d(inputL, "inputL");
@@ -437,6 +475,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("conv_inf_dist_forward_nograd", &conv_inf_dist_forward_nograd);
     m.def("conv_bound_inf_dist_forward_nograd", &conv_bound_inf_dist_forward_nograd);
     m.def("conv_inf_dist_forward", &conv_inf_dist_forward);
+    m.def("conv_norm_dist_forward", &conv_norm_dist_forward);
+    m.def("conv_norm_dist_backward_input", &conv_norm_dist_backward_input);
+    m.def("conv_norm_dist_backward_input_weight", &conv_norm_dist_backward_input_weight);
     m.def("conv_bound_inf_dist_forward", &conv_bound_inf_dist_forward);
     m.def("conv_inf_dist_backward_input", &conv_inf_dist_backward_input);
     m.def("conv_inf_dist_backward_input_weight", &conv_inf_dist_backward_input_weight);

@@ -249,7 +249,7 @@ size_t norm_backward_scratch_bytes(const Geom& s, float p) {
 }
 
 int launch_norm_backward(const float* gout, const float* x, const float* w, const float* out, const Geom& s, float* gx,
-                         float* gw, float p, hipStream_t st) {
+                         float* gw, float p, hipStream_t st, const UnfoldGeom* cv) {
     const float q = p - 1.0f;
     const BwdPlan pl = plan_backward(s, p);
     const int ip = pl.ip, cfg = pl.cfg;
@@ -281,7 +281,8 @@ int launch_norm_backward(const float* gout, const float* x, const float* w, cons
     }
     if (adaptive) {
         rc = fill_zero(aux, 8, st);
-        if (!rc) rc = launch_norm_probe(x, w, s, exp2f(-40.0f / q), reinterpret_cast<int*>(aux), st);
+        // (on images the probe runs below, on the patch rows)
+        if (!rc && cv == nullptr) rc = launch_norm_probe(x, w, s, exp2f(-40.0f / q), reinterpret_cast<int*>(aux), st);
         P.gmax = aux + 4;
         P.gate = reinterpret_cast<const int*>(aux);
         P.gate_limit = skip_override_limit(norm_probe_limit(s));
@@ -293,17 +294,40 @@ int launch_norm_backward(const float* gout, const float* x, const float* w, cons
         if (hip_failed(hipGetLastError())) rc = 4;
     }
     const long nx = (long)s.M * s.CIg * s.G;
-    bool transposed = s.HW >= kBwdTransposeMinHW && s.B <= 65535;
-    float* xT = nullptr;  // [M][CI] copy of x, followed by the [M][CI] gradient
+    // On images (cv): the patches are written straight into the row layout (or, for geometries that kernel does not
+    // take, extracted into a third buffer in the unfolded layout [B][CI][HW] and transposed like an unfolded input);
+    // the third buffer holds the unfolded gradient on its way back into the image.
+    bool transposed = cv != nullptr || (s.HW >= kBwdTransposeMinHW && s.B <= 65535);
+    float* xT = nullptr;  // [M][CI] copy of x, followed by the [M][CI] gradient (and the unfolded buffer)
+    float* unfolded = nullptr;
     if (!rc && transposed) {
-        if (scratch_alloc((void**)&xT, 2 * (size_t)nx * sizeof(float), st) != hipSuccess) {
+        const hipError_t e = scratch_alloc((void**)&xT, (cv != nullptr ? 3 : 2) * (size_t)nx * sizeof(float), st);
+        if (e != hipSuccess && cv != nullptr) {  // on images there is no other path
+            if (aux != nullptr) (void)scratch_free(aux, st);
+            (void)scratch_free(aT, st);
+            return hip_status(e);
+        }
+        if (e != hipSuccess) {
             (void)hipGetLastError();  // no room for the copies: the direct, uncoalesced path still works
             xT = nullptr;
             transposed = false;
         } else {
-            rc = transpose_batched(x, xT, s.B, s.CIg * s.G, s.HW, st);
+            const float* src = x;
+            bool rows_done = false;
+            if (cv != nullptr) {
+                unfolded = xT + 2 * nx;
+                rc = launch_patch_rows(x, *cv, xT, st);  // straight into the row layout where the geometry allows
+                rows_done = rc == 0;
+                if (rc == -1) {
+                    rc = launch_unfold(x, *cv, unfolded, st);
+                    src = unfolded;
+                }
+            }
+            if (!rc && !rows_done) rc = transpose_batched(src, xT, s.B, s.CIg * s.G, s.HW, st);
             P.s.B = s.M;
             P.s.HW = 1;
+            if (!rc && adaptive && cv != nullptr)
+                rc = launch_norm_probe(xT, w, P.s, exp2f(-40.0f / q), reinterpret_cast<int*>(aux), st);
         }
     }
     float* gx_k = transposed ? xT + nx : gx;
@@ -360,7 +384,8 @@ int launch_norm_backward(const float* gout, const float* x, const float* w, cons
                 break;
         }
     }
-    if (!rc && transposed) rc = transpose_batched(gx_k, gx, s.B, s.HW, s.CIg * s.G, st);
+    if (!rc && transposed) rc = transpose_batched(gx_k, cv != nullptr ? unfolded : gx, s.B, s.HW, s.CIg * s.G, st);
+    if (!rc && cv != nullptr) rc = launch_fold(unfolded, *cv, gx, st);
     if (xT != nullptr && hip_failed(scratch_free(xT, st)) && !rc) rc = 4;
     if (aux != nullptr && hip_failed(scratch_free(aux, st)) && !rc) rc = 4;
     if (hip_failed(scratch_free(aT, st)) && !rc) rc = 4;

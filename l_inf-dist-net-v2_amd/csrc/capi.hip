@@ -408,6 +408,53 @@ int ndist_conv_bound_inf_dist_forward(const float* inputL, const float* inputU, 
 // Backward of the fused layer.  The image-gradient kernels need one image plane (and one weight row) in LDS; other
 // geometries go the long way: gradient of the unfolded tensor in scratch memory, then the adjoint of
 // the patch extraction.
+int ndist_conv_norm_dist_forward(const float* input, const float* weight, int B, int C, int H, int W, int CO, int G,
+                                 int kernel_h, int kernel_w, int dilation_h, int dilation_w, int padding_h, int padding_w,
+                                 int stride_h, int stride_w, float* output, float p, ndist_stream_t stream) {
+    NDIST_REQUIRE(input); NDIST_REQUIRE(weight); NDIST_REQUIRE(output);
+    if (!finite_positive(p)) return NDIST_ERR_BAD_P;
+    UnfoldGeom u;
+    Geom s;
+    if (int rc = make_conv_geom(B, C, H, W, CO, G, kernel_h, kernel_w, dilation_h, dilation_w, padding_h, padding_w,
+                                stride_h, stride_w, &u, &s))
+        return rc;
+    return launch_norm_forward_conv(input, weight, s, output, p, (hipStream_t)stream, u);
+}
+
+static int conv_norm_backward(const float* grad_output, const float* input, const float* weight, const float* output,
+                              int B, int C, int H, int W, int CO, int G, int kernel_h, int kernel_w, int dilation_h,
+                              int dilation_w, int padding_h, int padding_w, int stride_h, int stride_w, float* grad_input,
+                              float* grad_weight, float p, ndist_stream_t stream) {
+    NDIST_REQUIRE(grad_output); NDIST_REQUIRE(input); NDIST_REQUIRE(weight); NDIST_REQUIRE(output);
+    NDIST_REQUIRE(grad_input);
+    if (!finite_positive(p)) return NDIST_ERR_BAD_P;
+    UnfoldGeom u;
+    Geom s;
+    if (int rc = make_conv_geom(B, C, H, W, CO, G, kernel_h, kernel_w, dilation_h, dilation_w, padding_h, padding_w,
+                                stride_h, stride_w, &u, &s))
+        return rc;
+    return launch_norm_backward(grad_output, input, weight, output, s, grad_input, grad_weight, p, (hipStream_t)stream,
+                                &u);
+}
+
+int ndist_conv_norm_dist_backward_input(const float* grad_output, const float* input, const float* weight,
+                                        const float* output, int B, int C, int H, int W, int CO, int G, int kernel_h,
+                                        int kernel_w, int dilation_h, int dilation_w, int padding_h, int padding_w,
+                                        int stride_h, int stride_w, float* grad_input, float p, ndist_stream_t stream) {
+    return conv_norm_backward(grad_output, input, weight, output, B, C, H, W, CO, G, kernel_h, kernel_w, dilation_h,
+                              dilation_w, padding_h, padding_w, stride_h, stride_w, grad_input, nullptr, p, stream);
+}
+
+int ndist_conv_norm_dist_backward_input_weight(const float* grad_output, const float* input, const float* weight,
+                                               const float* output, int B, int C, int H, int W, int CO, int G,
+                                               int kernel_h, int kernel_w, int dilation_h, int dilation_w, int padding_h,
+                                               int padding_w, int stride_h, int stride_w, float* grad_input,
+                                               float* grad_weight, float p, ndist_stream_t stream) {
+    NDIST_REQUIRE(grad_weight);
+    return conv_norm_backward(grad_output, input, weight, output, B, C, H, W, CO, G, kernel_h, kernel_w, dilation_h,
+                              dilation_w, padding_h, padding_w, stride_h, stride_w, grad_input, grad_weight, p, stream);
+}
+
 static int conv_backward(const float* g1, const float* g2, const int32_t* p1, const int32_t* p2, const UnfoldGeom& u,
                          const Geom& s, float* gx1, float* gx2, float* gw, hipStream_t st) {
     const bool bound = g2 != nullptr;

@@ -252,6 +252,8 @@ int bounds_override_limit(int probed_limit);
 void set_skip_mode(int skip, int bounds);
 int launch_unfold(const float* x, const UnfoldGeom& u, float* out, hipStream_t st);
 int launch_fold(const float* gout, const UnfoldGeom& u, float* gx, hipStream_t st);
+// the patches as rows [B * OH * OW][C * kh * kw] (the transpose of the unfolded tensor); -1: geometry not served
+int launch_patch_rows(const float* x, const UnfoldGeom& u, float* out, hipStream_t st);
 // The forward launchers take an optional patch geometry `cv`: x (xl, xu) are then images [B, C, H, W], s describes
 // the unfolded problem (CIg = C / G * kh * kw, HW = OH * OW) and the kernels extract the patches while loading.
 int launch_inf_forward(const float* x, const float* w, const Geom& s, float* out, int32_t* pos, hipStream_t st,
@@ -266,8 +268,13 @@ int launch_inf_bound_forward(const float* x, const float* xl, const float* xu, c
                              int32_t* pos, float* yl, float* yu, int32_t* pl, int32_t* pu, hipStream_t st);
 int launch_norm_forward(const float* x, const float* w, const float* max_in, const Geom& s, float* out, float p,
                         hipStream_t st);
+// on images: s describes the unfolded problem, the kernels extract the patches themselves
+int launch_norm_forward_conv(const float* x, const float* w, const Geom& s, float* out, float p, hipStream_t st,
+                             const UnfoldGeom& cv);
+// With a patch geometry x and gx are images [B, C, H, W] and s describes the unfolded problem: the patches go
+// straight into the row layout the kernel reads; the gradient rows are transposed and folded back into the image.
 int launch_norm_backward(const float* gout, const float* x, const float* w, const float* out, const Geom& s,
-                         float* gx, float* gw, float p, hipStream_t st);
+                         float* gx, float* gw, float p, hipStream_t st, const UnfoldGeom* cv = nullptr);
 // bytes of scratch launch_norm_backward cannot do without (the factor array); everything else it asks for is optional
 size_t norm_backward_scratch_bytes(const Geom& s, float p);
 // With a patch geometry the input gradients are images [B, C, H, W] (the adjoint of the patch extraction is applied

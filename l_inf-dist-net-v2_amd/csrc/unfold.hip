@@ -68,6 +68,74 @@ __global__ __launch_bounds__(256) void fold_kernel(const float* __restrict__ gou
     gx[e] = acc;
 }
 
+// The patches as rows: out[m][k] with m = (b, oh, ow) and k = (c, i, j), k contiguous -- the transpose of the unfolded
+// tensor, which is what the fused finite-p backward reads (lanes over k).  A workgroup owns one output row oh of one
+// sample and CC channels: it stages the kh image rows those patches read (whole rows, coalesced) in LDS as
+// strip[i][c][w], then writes, for every ow, the CC * kh * kw values of the row as one contiguous run.  Index
+// arithmetic by float-reciprocal divisions (all operands below 2^22, checked by the launcher).
+__global__ __launch_bounds__(256) void patch_rows_kernel(const float* __restrict__ x, float* __restrict__ out,
+                                                         const UnfoldGeom u, int CC, int ncb, int vec4, float inv_w,
+                                                         float inv_ccw, float inv_taps, float inv_kw) {
+    extern __shared__ float strip[];  // [kh][CC][WP], WP = W | 1: neighbouring channels in different banks
+    const int WP = u.W | 1;
+    unsigned id = blockIdx.x;
+    const int cb = (int)(id % (unsigned)ncb);
+    id /= (unsigned)ncb;
+    const int oh = (int)(id % (unsigned)u.OH), b = (int)(id / (unsigned)u.OH);
+    const int c0 = cb * CC, ncl = min(CC, u.C - c0);
+    const int taps = u.kh * u.kw, L = u.OH * u.OW;
+    const long K = (long)u.C * taps;
+    const int ccw = CC * u.W;
+    for (int idx = threadIdx.x; idx < u.kh * ccw; idx += 256) {
+        const int i = small_div(idx, ccw, inv_ccw), rem = idx - i * ccw;
+        const int cl = small_div(rem, u.W, inv_w), wc = rem - cl * u.W;
+        const int h = oh * u.sh - u.ph + i * u.dh;
+        strip[(i * CC + cl) * WP + wc] =
+            (cl < ncl && (unsigned)h < (unsigned)u.H) ? x[(((long)b * u.C + c0 + cl) * u.H + h) * u.W + wc] : 0.f;
+    }
+    __syncthreads();
+    const int run = ncl * taps;  // contiguous floats per output position
+    float* __restrict__ dst = out + ((long)b * L + (long)oh * u.OW) * K + (long)c0 * taps;
+    auto value = [&](int ow, int kk) {
+        const int cl = small_div(kk, taps, inv_taps), tap = kk - cl * taps;
+        const int i = small_div(tap, u.kw, inv_kw), j = tap - i * u.kw;
+        const int wc = ow * u.sw - u.pw + j * u.dw;
+        return (unsigned)wc < (unsigned)u.W ? strip[(i * CC + cl) * WP + wc] : 0.f;
+    };
+    if (vec4) {  // run and K are multiples of four and out is 16-byte aligned: one store per four values
+        const int run4 = run >> 2;
+        const float inv_run4 = 1.0f / (float)run4;
+        for (int idx = threadIdx.x; idx < u.OW * run4; idx += 256) {
+            const int ow = small_div(idx, run4, inv_run4), kk = (idx - ow * run4) * 4;
+            *reinterpret_cast<float4*>(dst + (long)ow * K + kk) =
+                make_float4(value(ow, kk), value(ow, kk + 1), value(ow, kk + 2), value(ow, kk + 3));
+        }
+    } else {
+        const float inv_run = 1.0f / (float)run;
+        for (int idx = threadIdx.x; idx < u.OW * run; idx += 256) {
+            const int ow = small_div(idx, run, inv_run), kk = idx - ow * run;
+            dst[(long)ow * K + kk] = value(ow, kk);
+        }
+    }
+}
+
+// returns -1 (nothing launched) when the geometry does not fit the kernel: the caller unfolds and transposes then
+int launch_patch_rows(const float* x, const UnfoldGeom& u, float* out, hipStream_t st) {
+    const int taps = u.kh * u.kw;
+    int CC = 8192 / (u.kh * (u.W | 1));  // 32 KB of LDS for the strip
+    CC = CC > u.C ? u.C : CC;
+    if (CC < 1 || (long)u.kh * CC * u.W >= (1L << 22) || (long)u.OW * CC * taps >= (1L << 22)) return -1;
+    const int ncb = (u.C + CC - 1) / CC;
+    const long blocks = (long)u.B * u.OH * ncb;
+    if (blocks >= (1L << 31)) return -1;
+    // 16-byte stores need every run of a workgroup to start and end on a multiple of four floats
+    const int vec4 = (CC * taps) % 4 == 0 && (u.C * taps) % 4 == 0 && (uintptr_t)out % 16 == 0;
+    hipLaunchKernelGGL(patch_rows_kernel, dim3((unsigned)blocks), dim3(256), (size_t)u.kh * CC * (u.W | 1) * sizeof(float), st, x,
+                       out, u, CC, ncb, vec4, 1.0f / (float)u.W, 1.0f / (float)(CC * u.W), 1.0f / (float)taps,
+                       1.0f / (float)u.kw);
+    return hip_failed(hipGetLastError()) ? 4 : 0;
+}
+
 int launch_unfold(const float* x, const UnfoldGeom& u, float* out, hipStream_t st) {
     const int L = u.OH * u.OW;
     const bool vec = L % 4 == 0 && (uintptr_t)out % 16 == 0;
