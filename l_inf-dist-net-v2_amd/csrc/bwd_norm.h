@@ -49,6 +49,12 @@ struct BwdParams {
     const int* gate2;
     int gate2_limit, gate2_sense;
     long g_off;       // unfolded variant only: offset in floats from the 1/out factors to the grad_output factors
+    // Reproducible grad_input (row-split kernel): a workgroup that holds ALL units of a (group, slab, row chunk) block
+    // stores that block's grad_input directly; a block shared between neighbouring workgroups goes into `part`
+    // ([workgroup][2][rows per workgroup][64]: slot 0 for the block a workgroup starts in, slot 1 for the one it ends
+    // in) and bwd_gx_fixup_kernel adds the shares in workgroup order.  nullptr: global atomic adds into a zeroed
+    // grad_input (sums in arrival order).
+    float* part;
 };
 
 typedef float f16v __attribute__((ext_vector_type(16)));
@@ -264,12 +270,23 @@ __global__ __launch_bounds__(64 * NW, 4) void bwd_fused_kernel(const float* __re
 
     auto flush_gx = [&]() {
         if (!x_ok) return;
+        const long b0 = loaded_sr * P.ncc;
+        const bool sole = P.part != nullptr && u_begin <= b0 && b0 + P.ncc <= u_end;  // all units of the block are mine
+        if (P.part != nullptr && !sole) {
+            const int slot = loaded_sr == u_begin / P.ncc ? 0 : 1;
+            float* __restrict__ dst = P.part + (((long)blockIdx.x * 2 + slot) * (NW * BT) + wave * BT) * kBwdSlab + lane;
+#pragma unroll
+            for (int i = 0; i < BT; i++) dst[i * kBwdSlab] = gxa[i];
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < BT; i++) {
             const int m = xr0 + i;
             if (m < s.M) {
                 const int b = m / s.HW, hw = m - b * s.HW;
-                atomicAdd(GX + x_off(s, b, xg, xci, hw), gxa[i]);
+                float* __restrict__ dst = GX + x_off(s, b, xg, xci, hw);
+                if (sole) *dst = gxa[i];
+                else atomicAdd(dst, gxa[i]);
             }
         }
     };

@@ -34,6 +34,44 @@ template <> int launch_bwd_ip<-4>(const BwdPtrs& a, const BwdParams& P, int cfg,
     return hip_failed(hipGetLastError()) ? 4 : 0;
 }
 
+// Second step of the reproducible grad_input, over the (group, slab, row chunk) blocks.  The persistent
+// workgroups of the main kernel took the unit ranges [g * total / nwg, (g + 1) * total / nwg); a block whose units lie
+// in one range was stored by that workgroup, every other block is the sum, in workgroup order, of the shares its
+// workgroups left in `part`.
+__global__ __launch_bounds__(256) void bwd_gx_fixup_kernel(const float* __restrict__ part, float* __restrict__ GX,
+                                                           const BwdParams P, int nwg, int rows_per_wg) {
+    const Geom& s = P.s;
+    // (1024 elements of a block per workgroup)
+    const int nchunk = (rows_per_wg * kBwdSlab + 1023) / 1024;
+    const long sr = blockIdx.x / (unsigned)nchunk, b0 = sr * P.ncc, b1 = b0 + P.ncc;
+    const int e0 = (int)(blockIdx.x % (unsigned)nchunk) * 1024;
+    auto begin = [&](long g) { return g * P.total / nwg; };
+    auto owner = [&](long u) {  // the workgroup whose range holds unit u
+        long g = u * nwg / P.total;
+        g = g < 0 ? 0 : (g > nwg - 1 ? nwg - 1 : g);
+        while (g > 0 && begin(g) > u) g--;
+        while (g + 1 < nwg && begin(g + 1) <= u) g++;
+        return g;
+    };
+    const long g_lo = owner(b0), g_hi = owner(b1 - 1);
+    if (g_lo == g_hi) return;
+    const int rc = (int)(sr % P.nrc);
+    const int gs = (int)(sr / P.nrc);
+    const int grp = gs / P.nslab, ci0 = (gs - grp * P.nslab) * kBwdSlab;
+    for (int e = e0 + threadIdx.x; e < min(e0 + 1024, rows_per_wg * kBwdSlab); e += 256) {
+        const int r = e / kBwdSlab, l = e - r * kBwdSlab;
+        const int m = rc * rows_per_wg + r, ci = ci0 + l;
+        if (m >= s.M || ci >= s.CIg) continue;
+        float v = 0.f;
+        for (long g = g_lo; g <= g_hi; g++) {
+            const int slot = sr == begin(g) / P.ncc ? 0 : 1;
+            v += part[((g * 2 + slot) * rows_per_wg + r) * kBwdSlab + l];
+        }
+        const int b = m / s.HW, hw = m - b * s.HW;
+        GX[x_off(s, b, grp, ci, hw)] = v;
+    }
+}
+
 // pre-pass: the per-(row, co) factor, transposed to [gco][m]
 //   p = 1: grad_output ;  p >= 2: sign(g) * |g|^(1/(p-1)) / out  (root in double precision: its error is multiplied
 //   by p-1 when the main kernel raises the factor to that power again) ;  1 < p < 2 (g_off != 0): 1/out, and
@@ -331,14 +369,28 @@ int launch_norm_backward(const float* gout, const float* x, const float* w, cons
         }
     }
     float* gx_k = transposed ? xT + nx : gx;
-    if (!rc) rc = fill_zero(gx_k, nx, st);
+    // Reproducible grad_input: shares of the blocks that two workgroups split go through a buffer and are added in a
+    // fixed order (see BwdParams::part).  Not for the small-batch kernel, not where several kernel variants are
+    // queued (their grids may differ), not from the fixed scratch array (64 MB at the headline shape): those add
+    // with atomics into a zeroed gradient.
+    const long cap = (long)device_info().num_cu * (cfg == 1 ? 2 : (cfg == 2 ? 4 : (cfg == 4 ? 6 : 1)));
+    const int grid = (int)(P.total < cap ? P.total : cap);
+    float* part = nullptr;
+    // (NORM_DIST_BWD_ATOMIC=1: tuning aid, the atomic adds everywhere)
+    static const bool force_atomic = getenv("NORM_DIST_BWD_ATOMIC") != nullptr && getenv("NORM_DIST_BWD_ATOMIC")[0] == '1';
+    if (!rc && cfg != 3 && !adaptive && !static_scratch_active() && !force_atomic) {
+        if (scratch_alloc((void**)&part, 2 * (size_t)grid * rows_per_wg * kBwdSlab * sizeof(float), st) != hipSuccess) {
+            (void)hipGetLastError();
+            part = nullptr;
+        }
+    }
+    P.part = part;
+    if (!rc && part == nullptr) rc = fill_zero(gx_k, nx, st);
     if (!rc && gw != nullptr && P.nrc > 1) rc = fill_zero(gw, (long)s.COg * s.G * s.CIg, st);
     if (!rc) {
         // Persistent workgroups take equal shares of the units, so all of them should be resident at once: two 8-wave
         // workgroups fit a compute unit (72 KB of LDS each), four 4-wave ones (40 KB each, exactly the 160 KB) and six
         // 2-wave ones (24.6 KB each).
-        const long cap = (long)device_info().num_cu * (cfg == 1 ? 2 : (cfg == 2 ? 4 : (cfg == 4 ? 6 : 1)));
-        const int grid = (int)(P.total < cap ? P.total : cap);
         BwdPtrs a{transposed ? xT : x, w, aT, gx_k, gw};
         switch (ip) {
             case 0: rc = launch_bwd_ip<0>(a, P, cfg, grid, st); break;
@@ -384,6 +436,12 @@ int launch_norm_backward(const float* gout, const float* x, const float* w, cons
                 break;
         }
     }
+    if (!rc && part != nullptr) {
+        const long nblk = (long)s.G * P.nslab * P.nrc * ((rows_per_wg * kBwdSlab + 1023) / 1024);
+        hipLaunchKernelGGL(bwd_gx_fixup_kernel, dim3((unsigned)nblk), dim3(256), 0, st, part, gx_k, P, grid, rows_per_wg);
+        if (hip_failed(hipGetLastError())) rc = 4;
+    }
+    if (part != nullptr && hip_failed(scratch_free(part, st)) && !rc) rc = 4;
     if (!rc && transposed) rc = transpose_batched(gx_k, cv != nullptr ? unfolded : gx, s.B, s.HW, s.CIg * s.G, st);
     if (!rc && cv != nullptr) rc = launch_fold(unfolded, *cv, gx, st);
     if (xT != nullptr && hip_failed(scratch_free(xT, st)) && !rc) rc = 4;
