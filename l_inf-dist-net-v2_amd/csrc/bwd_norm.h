@@ -270,14 +270,20 @@ __global__ __launch_bounds__(64 * NW, 4) void bwd_fused_kernel(const float* __re
 
     auto flush_gx = [&]() {
         if (!x_ok) return;
-        const long b0 = loaded_sr * P.ncc;
-        const bool sole = P.part != nullptr && u_begin <= b0 && b0 + P.ncc <= u_end;  // all units of the block are mine
-        if (P.part != nullptr && !sole) {
-            const int slot = loaded_sr == u_begin / P.ncc ? 0 : 1;
-            float* __restrict__ dst = P.part + (((long)blockIdx.x * 2 + slot) * (NW * BT) + wave * BT) * kBwdSlab + lane;
+        // (the skipping variants are only ever queued next to other variants, where `part` is not used: they keep
+        // the plain atomic path, and their register budget)
+        constexpr bool kShares = IP != -3 && IP != -4;
+        bool sole = false;
+        if constexpr (kShares) {
+            const long b0 = loaded_sr * P.ncc;
+            sole = P.part != nullptr && u_begin <= b0 && b0 + P.ncc <= u_end;  // all units of the block are mine
+            if (P.part != nullptr && !sole) {
+                const int slot = loaded_sr == u_begin / P.ncc ? 0 : 1;
+                float* __restrict__ dst = P.part + (((long)blockIdx.x * 2 + slot) * (NW * BT) + wave * BT) * kBwdSlab + lane;
 #pragma unroll
-            for (int i = 0; i < BT; i++) dst[i * kBwdSlab] = gxa[i];
-            return;
+                for (int i = 0; i < BT; i++) dst[i * kBwdSlab] = gxa[i];
+                return;
+            }
         }
 #pragma unroll
         for (int i = 0; i < BT; i++) {
