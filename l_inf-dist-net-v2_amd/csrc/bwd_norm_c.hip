@@ -334,12 +334,13 @@ int launch_norm_backward(const float* gout, const float* x, const float* w, cons
     const long nx = (long)s.M * s.CIg * s.G;
     // On images (cv): the patches are written straight into the row layout (or, for geometries that kernel does not
     // take, extracted into a third buffer in the unfolded layout [B][CI][HW] and transposed like an unfolded input);
-    // the third buffer holds the unfolded gradient on its way back into the image.
+    // the gradient rows are folded back into the image by one gather.
     bool transposed = cv != nullptr || (s.HW >= kBwdTransposeMinHW && s.B <= 65535);
     float* xT = nullptr;  // [M][CI] copy of x, followed by the [M][CI] gradient (and the unfolded buffer)
     float* unfolded = nullptr;
     if (!rc && transposed) {
-        const hipError_t e = scratch_alloc((void**)&xT, (cv != nullptr ? 3 : 2) * (size_t)nx * sizeof(float), st);
+        const bool via_unfold = cv != nullptr && !patch_rows_applies(*cv);  // needs the third buffer
+        const hipError_t e = scratch_alloc((void**)&xT, (via_unfold ? 3 : 2) * (size_t)nx * sizeof(float), st);
         if (e != hipSuccess && cv != nullptr) {  // on images there is no other path
             if (aux != nullptr) (void)scratch_free(aux, st);
             (void)scratch_free(aT, st);
@@ -352,14 +353,13 @@ int launch_norm_backward(const float* gout, const float* x, const float* w, cons
         } else {
             const float* src = x;
             bool rows_done = false;
-            if (cv != nullptr) {
+            if (cv != nullptr && !via_unfold) {
+                rc = launch_patch_rows(x, *cv, xT, st);  // straight into the row layout
+                rows_done = true;
+            } else if (cv != nullptr) {
                 unfolded = xT + 2 * nx;
-                rc = launch_patch_rows(x, *cv, xT, st);  // straight into the row layout where the geometry allows
-                rows_done = rc == 0;
-                if (rc == -1) {
-                    rc = launch_unfold(x, *cv, unfolded, st);
-                    src = unfolded;
-                }
+                rc = launch_unfold(x, *cv, unfolded, st);
+                src = unfolded;
             }
             if (!rc && !rows_done) rc = transpose_batched(src, xT, s.B, s.CIg * s.G, s.HW, st);
             P.s.B = s.M;
@@ -442,8 +442,8 @@ int launch_norm_backward(const float* gout, const float* x, const float* w, cons
         if (hip_failed(hipGetLastError())) rc = 4;
     }
     if (part != nullptr && hip_failed(scratch_free(part, st)) && !rc) rc = 4;
-    if (!rc && transposed) rc = transpose_batched(gx_k, cv != nullptr ? unfolded : gx, s.B, s.HW, s.CIg * s.G, st);
-    if (!rc && cv != nullptr) rc = launch_fold(unfolded, *cv, gx, st);
+    if (!rc && cv != nullptr) rc = launch_fold_rows(gx_k, *cv, gx, st);
+    else if (!rc && transposed) rc = transpose_batched(gx_k, gx, s.B, s.HW, s.CIg * s.G, st);
     if (xT != nullptr && hip_failed(scratch_free(xT, st)) && !rc) rc = 4;
     if (aux != nullptr && hip_failed(scratch_free(aux, st)) && !rc) rc = 4;
     if (hip_failed(scratch_free(aT, st)) && !rc) rc = 4;

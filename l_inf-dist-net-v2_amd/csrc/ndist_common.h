@@ -254,6 +254,9 @@ int launch_unfold(const float* x, const UnfoldGeom& u, float* out, hipStream_t s
 int launch_fold(const float* gout, const UnfoldGeom& u, float* gx, hipStream_t st);
 // the patches as rows [B * OH * OW][C * kh * kw] (the transpose of the unfolded tensor); -1: geometry not served
 int launch_patch_rows(const float* x, const UnfoldGeom& u, float* out, hipStream_t st);
+bool patch_rows_applies(const UnfoldGeom& u);
+// the adjoint: image gradient from gradient rows [B * OH * OW][C * kh * kw] (any geometry)
+int launch_fold_rows(const float* g, const UnfoldGeom& u, float* gx, hipStream_t st);
 // The forward launchers take an optional patch geometry `cv`: x (xl, xu) are then images [B, C, H, W], s describes
 // the unfolded problem (CIg = C / G * kh * kw, HW = OH * OW) and the kernels extract the patches while loading.
 int launch_inf_forward(const float* x, const float* w, const Geom& s, float* out, int32_t* pos, hipStream_t st,
@@ -272,7 +275,7 @@ int launch_norm_forward(const float* x, const float* w, const float* max_in, con
 int launch_norm_forward_conv(const float* x, const float* w, const Geom& s, float* out, float p, hipStream_t st,
                              const UnfoldGeom& cv);
 // With a patch geometry x and gx are images [B, C, H, W] and s describes the unfolded problem: the patches go
-// straight into the row layout the kernel reads; the gradient rows are transposed and folded back into the image.
+// straight into the row layout the kernel reads and the gradient rows are folded back into the image.
 int launch_norm_backward(const float* gout, const float* x, const float* w, const float* out, const Geom& s,
                          float* gx, float* gw, float p, hipStream_t st, const UnfoldGeom* cv = nullptr);
 // bytes of scratch launch_norm_backward cannot do without (the factor array); everything else it asks for is optional

@@ -119,6 +119,76 @@ __global__ __launch_bounds__(256) void patch_rows_kernel(const float* __restrict
     }
 }
 
+// Adjoint of the above: gx[b, c, h, w] = sum over the taps (i, j) that read this pixel of g[m(b, oh, ow)][(c, i, j)].
+// A workgroup owns 64 channels x 32 pixels of one image row; its threads run over the channels first, so that the
+// reads of one tap (36 bytes apart for a 3 x 3 window) and of the neighbouring pixels' taps fall into the same cache
+// lines, and the sums turn around in LDS for writes that run along w.  UNIT: both strides are 1 (no divisions).
+// The taps are added in a fixed order: reproducible.
+template <bool UNIT>
+__global__ __launch_bounds__(256) void fold_rows_kernel(const float* __restrict__ g, float* __restrict__ gx,
+                                                        const UnfoldGeom u) {
+    __shared__ float tile[64][33];
+    const int nwb = (u.W + 31) / 32, ncb = (u.C + 63) / 64;
+    unsigned id = blockIdx.x;
+    const int wb = (int)(id % (unsigned)nwb);
+    id /= (unsigned)nwb;
+    const int cb = (int)(id % (unsigned)ncb);
+    id /= (unsigned)ncb;
+    const int h = (int)(id % (unsigned)u.H), b = (int)(id / (unsigned)u.H);
+    const int taps = u.kh * u.kw, L = u.OH * u.OW;
+    const long K = (long)u.C * taps;
+    const int cl = threadIdx.x & 63, c = cb * 64 + cl;
+    const float* __restrict__ gb = g + (long)b * L * K + (long)(c < u.C ? c : 0) * taps;
+    for (int wl = threadIdx.x >> 6; wl < 32; wl += 4) {
+        const int w = wb * 32 + wl;
+        float acc = 0.f;
+        if (c < u.C && w < u.W) {
+            for (int i = 0; i < u.kh; i++) {
+                const int hn = h + u.ph - i * u.dh;
+                int oh = hn;
+                if (!UNIT) {
+                    if (hn < 0 || hn % u.sh != 0) continue;
+                    oh = hn / u.sh;
+                }
+                if ((unsigned)oh >= (unsigned)u.OH) continue;
+                for (int j = 0; j < u.kw; j++) {
+                    const int wn = w + u.pw - j * u.dw;
+                    int ow = wn;
+                    if (!UNIT) {
+                        if (wn < 0 || wn % u.sw != 0) continue;
+                        ow = wn / u.sw;
+                    }
+                    if ((unsigned)ow >= (unsigned)u.OW) continue;
+                    acc += gb[(long)(oh * u.OW + ow) * K + i * u.kw + j];
+                }
+            }
+        }
+        tile[cl][wl] = acc;
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < 64 * 32; idx += 256) {
+        const int cc = idx >> 5, wl = idx & 31;
+        const int c2 = cb * 64 + cc, w = wb * 32 + wl;
+        if (c2 < u.C && w < u.W) gx[(((long)b * u.C + c2) * u.H + h) * u.W + w] = tile[cc][wl];
+    }
+}
+
+int launch_fold_rows(const float* g, const UnfoldGeom& u, float* gx, hipStream_t st) {
+    const long blocks = (long)u.B * u.H * ((u.C + 63) / 64) * ((u.W + 31) / 32);
+    if (blocks >= (1L << 31)) return 2;
+    if (u.sh == 1 && u.sw == 1) hipLaunchKernelGGL(fold_rows_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, st, g, gx, u);
+    else hipLaunchKernelGGL(fold_rows_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, st, g, gx, u);
+    return hip_failed(hipGetLastError()) ? 4 : 0;
+}
+
+bool patch_rows_applies(const UnfoldGeom& u) {
+    const int taps = u.kh * u.kw;
+    int CC = 8192 / (u.kh * (u.W | 1));
+    CC = CC > u.C ? u.C : CC;
+    if (CC < 1 || (long)u.kh * CC * u.W >= (1L << 22) || (long)u.OW * CC * taps >= (1L << 22)) return false;
+    return (long)u.B * u.OH * ((u.C + CC - 1) / CC) < (1L << 31);
+}
+
 // returns -1 (nothing launched) when the geometry does not fit the kernel: the caller unfolds and transposes then
 int launch_patch_rows(const float* x, const UnfoldGeom& u, float* out, hipStream_t st) {
     const int taps = u.kh * u.kw;
