@@ -75,7 +75,8 @@ __device__ __forceinline__ void hot_group_maxima(const float* __restrict__ seed_
 
 // One kernel for the whole plan.  Every workgroup (1024 threads) first finds MX and MW of all groups, then its 16
 // waves turn four rows each (rows of x first, then rows of w; their loads issued together) into hot-tile masks: bit
-// t of a row's mask = tile t is hot.  The workgroups leave their counts of hot (row, tile) entries per side in
+// t of a row's mask = tile t is hot (a row's record: one word naming its non-zero mask words, then the mask words).
+// The workgroups leave their counts of hot (row, tile) entries per side in
 // `partial`; the last one to finish (a ticket in dec[3], cleared by the row pre-pass) adds them up and decides:
 //   dec[0] = 1: the rows of x select the tiles, 2: the rows of w, 0: too many hot tiles, the dense kernels run.
 // Cost of a side = its hot entries x the length of the other side.  mode: 1 always the cheaper side, 2 / 3 always
@@ -103,6 +104,7 @@ __global__ __launch_bounds__(1024) void hot_plan_kernel(const float* __restrict_
     bool valid[R], isw[R];
     long rr[R];
     int count[R];
+    uint32_t nonzero[R];  // bit i: mask word i of the row has a hot tile (first word of the row's record)
 #pragma unroll
     for (int i = 0; i < R; i++) {
         const long r = (long)blockIdx.x * kPlanRows + wave * R + i;
@@ -120,8 +122,9 @@ __global__ __launch_bounds__(1024) void hot_plan_kernel(const float* __restrict_
             thr[i] = own == own ? (tu < tl ? tu : tl) : -__builtin_inf();
         }
         tm[i] = (isw[i] ? tile_w : tile_x) + rr[i] * ntile;
-        mk[i] = (isw[i] ? mask_w : mask_x) + rr[i] * nword;
+        mk[i] = (isw[i] ? mask_w : mask_x) + rr[i] * (nword + 1);
         count[i] = 0;
+        nonzero[i] = 0u;
     }
     for (int t0 = 0; t0 < nword * 32; t0 += 64) {
         const int t = t0 + lane;
@@ -133,9 +136,11 @@ __global__ __launch_bounds__(1024) void hot_plan_kernel(const float* __restrict_
             const bool hot = valid[i] && t < ntile && !((double)v[i] < thr[i]);
             const unsigned long long bits = __builtin_amdgcn_ballot_w64(hot);
             count[i] += __popcll(bits);
+            const int wi = t0 >> 5;
+            nonzero[i] |= ((uint32_t)bits != 0u ? 1u << (wi & 31) : 0u) | ((bits >> 32) != 0ull ? 1u << ((wi + 1) & 31) : 0u);
             if (lane == 0 && valid[i]) {
-                mk[i][t0 >> 5] = (uint32_t)bits;
-                if ((t0 >> 5) + 1 < nword) mk[i][(t0 >> 5) + 1] = (uint32_t)(bits >> 32);
+                mk[i][1 + wi] = (uint32_t)bits;
+                if (wi + 1 < nword) mk[i][2 + wi] = (uint32_t)(bits >> 32);
             }
         }
     }
@@ -143,6 +148,7 @@ __global__ __launch_bounds__(1024) void hot_plan_kernel(const float* __restrict_
 #pragma unroll
         for (int i = 0; i < R; i++) {
             if (!valid[i]) continue;
+            mk[i][0] = nonzero[i];
             if (count[i] != 0) atomicAdd(&cnt[isw[i] ? 1 : 0], count[i]);
         }
     }
@@ -283,8 +289,19 @@ __device__ __forceinline__ void hot_walk(const float* __restrict__ own, const fl
         const int row = q + 8 * j;
         rowp[j] = oth + (long)(row < nrow ? row : 0) * stride;
     }
-    for (int wi = 0; wi < nword; wi++) {
-        uint32_t bits = mk[wi];
+    // mk[0] names the mask words that hold a hot tile (when there are at most 32 of them): usually a single one, so
+    // the walk costs two dependent loads instead of one per word
+    uint32_t pending = mk[0];
+    int wi = -1;
+    while (true) {
+        if (nword <= 32) {
+            if (pending == 0) break;
+            wi = __builtin_ctz(pending);
+            pending &= pending - 1;
+        } else if (++wi >= nword) {
+            break;
+        }
+        uint32_t bits = mk[1 + wi];
         while (bits != 0) {
             const int k0 = (wi * 32 + __builtin_ctz(bits)) * 32 + 4 * sub;
             bits &= bits - 1;
@@ -371,7 +388,7 @@ __global__ __launch_bounds__(256) void hot_kernel(const float* __restrict__ x, l
         if (n0 >= s.COg) return;  // whole waves
         const int g = (int)(r % s.G);
         hot_walk<P, true>(x + r * s.CIg, w + ((long)g * s.COg + n0) * s.CIg, x2off, s.CIg, min(kHotRows, s.COg - n0),
-                          mask_x + r * nword, nword, s.CIg, vec != 0, res);
+                          mask_x + r * (nword + 1), nword, s.CIg, vec != 0, res);
         const int n = n0 + mine;
         if (reports && n < s.COg) {
             P::outputs(res, fv, iv);
@@ -395,7 +412,7 @@ __global__ __launch_bounds__(256) void hot_kernel(const float* __restrict__ x, l
             if (n < s.COg) {  // wave-uniform
                 const long wrow = (long)g * s.COg + n;
                 hot_walk<P, false>(w + wrow * s.CIg, x + ((long)m0 * s.G + g) * s.CIg, x2off, (long)s.CIg * s.G,
-                                   min(kHotRows, s.M - m0), mask_w + wrow * nword, nword, s.CIg, vec != 0, res);
+                                   min(kHotRows, s.M - m0), mask_w + wrow * (nword + 1), nword, s.CIg, vec != 0, res);
             }
             P::outputs(res, fv, iv);
             if (reports) {
@@ -442,7 +459,7 @@ bool hot_forward_applies(const Geom& s) { return hot_mode() != 0 && s.HW == 1 &&
 
 size_t hot_scratch_floats(const Geom& s) {
     const size_t nword = (size_t)ceil_div(ceil_div(s.CIg, 32), 32);
-    return 8 + 2 * (size_t)plan_blocks(s) + nword * ((size_t)s.M * s.G + (size_t)s.COg * s.G);
+    return 8 + 2 * (size_t)plan_blocks(s) + (nword + 1) * ((size_t)s.M * s.G + (size_t)s.COg * s.G);
 }
 
 static int launch_hot(const float* x, const float* x2, const float* w, const Geom& s, const SeedBuffers& sb, float* base,
@@ -452,7 +469,7 @@ static int launch_hot(const float* x, const float* x2, const float* w, const Geo
     int* dec = reinterpret_cast<int*>(base);  // [0] decision, [1], [2] hot entries per side, [3] ticket (cleared by the row pre-pass)
     int* partial = dec + 8;
     uint32_t* mask_x = reinterpret_cast<uint32_t*>(partial + 2 * nblk);
-    uint32_t* mask_w = mask_x + rows * nword;
+    uint32_t* mask_w = mask_x + rows * (nword + 1);
     *decision = dec;
     // at most 1 / 12 of all (row, column, tile) triples: measured at 5120 x 5120 with 512 and with 64 rows, the dense
     // kernels are the faster ones from about a tenth on
