@@ -204,6 +204,22 @@ int ndist_mean_shift_backward(const float* grad_y, const float* grad_y_lower, co
                               int HW, int training, float* grad_x, float* colsum_out, float* mean_scratch,
                               ndist_stream_t stream);
 
+/* Tail of a distance network, no kernels of their own in the reference either (ell_inf_models.py:41-46 and
+ * main.py:304-310 in torch primitives): the worst-case margins
+ *   margin[b, c] = (upper[b, t_b] - lower[b, c]) / (2 eps) for c != t_b, 0 for c == t_b        (t = targets, int64)
+ * of the logits -x (lower / upper NULL: x - eps / x + eps, the network being 1-Lipschitz in the infinity norm), and
+ * the hinge loss on them, loss = (1 - mix) * mean_b max_c relu(margin) + mix * mean relu(margin).  All tensors
+ * [B, C] contiguous; argmax [B] int32 links ndist_hinge_forward to its backward; loss and grad_loss are one float on
+ * the device.  The backward entry points overwrite their outputs (grad_x, or grad_lower and grad_upper; pass NULL
+ * for those that do not exist).  Sums in a fixed order. */
+int ndist_margin_forward(const float* x, const float* lower, const float* upper, const long long* targets, int B, int C,
+                         float eps, float* margin, ndist_stream_t stream);
+int ndist_margin_backward(const float* grad_margin, const long long* targets, int B, int C, float eps, float* grad_x,
+                          float* grad_lower, float* grad_upper, ndist_stream_t stream);
+int ndist_hinge_forward(const float* margin, int B, int C, float mix, float* loss, int* argmax, ndist_stream_t stream);
+int ndist_hinge_backward(const float* margin, const int* argmax, const float* grad_loss, int B, int C, float mix,
+                         float* grad_margin, ndist_stream_t stream);
+
 /* ---- patch extraction for the convolutional layer -------------------------------------------------------------
  * The reference has no kernel of its own here: NormDistConv calls torch.nn.functional.unfold
  * (core/modules/norm_dist.py:93-102).  These two entry points replace that call and its autograd adjoint with one

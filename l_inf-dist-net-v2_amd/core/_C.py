@@ -86,6 +86,10 @@ _bnd_bwd_xw = _sig("ndist_bound_inf_dist_backward_input_weight", _P, _P, _P, _P,
 _joint_ng = _sig("ndist_inf_and_bound_forward_nograd", _P, _P, _P, _P, *_DIMS, _P, _P, _P, _P)
 _joint = _sig("ndist_inf_and_bound_forward", _P, _P, _P, _P, *_DIMS, _P, _P, _P, _P, _P, _P, _P)
 _ms_fwd = _sig("ndist_mean_shift_forward", _P, _P, _P, _I, _I, _I, _I, _F, _P, _P, _P, _P, _P, _P, _P, _P)
+_margin_fwd = _sig("ndist_margin_forward", _P, _P, _P, _P, _I, _I, _F, _P, _P)
+_margin_bwd = _sig("ndist_margin_backward", _P, _P, _I, _I, _F, _P, _P, _P, _P)
+_hinge_fwd = _sig("ndist_hinge_forward", _P, _I, _I, _F, _P, _P, _P)
+_hinge_bwd = _sig("ndist_hinge_backward", _P, _P, _P, _I, _I, _F, _P, _P)
 _ms_bwd = _sig("ndist_mean_shift_backward", _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P)
 _unfold_fwd = _sig("ndist_unfold_forward", _P, *([_I] * 12), _P, _P)
 _unfold_bwd = _sig("ndist_unfold_backward", _P, *([_I] * 12), _P, _P)
@@ -396,6 +400,39 @@ def mean_shift_backward(grad_y, grad_y_lower, grad_y_upper, training, grad_x, co
                       colsum_out=colsum_out, mean_scratch=mean_scratch)
     _run(_ms_bwd, dev, _po(grad_y), _po(grad_y_lower), _po(grad_y_upper), B, C, HW, 1 if training else 0, _po(grad_x),
          _po(colsum_out), _po(mean_scratch))
+
+
+_TAIL = {"targets": torch.int64, "argmax": torch.int32}
+
+
+def margin_forward(x, lower, upper, targets, eps, margin):
+    """Worst-case margins of the logits -x (ell_inf_models.py:41-46): margin[b, c] = (upper[b, t_b] - lower[b, c]) /
+    (2 eps), 0 at c = t_b; lower / upper None: x -/+ eps.  (These four go through the C ABI with ctypes on either
+    binding: a handful of launches per step.)"""
+    dev = _check(_TAIL, **{k: v for k, v in dict(x=x, lower=lower, upper=upper, targets=targets, margin=margin).items()
+                           if v is not None})
+    B, C = margin.shape
+    _run(_margin_fwd, dev, _po(x), _po(lower), _po(upper), _p(targets), B, C, float(eps), _p(margin))
+
+
+def margin_backward(grad_margin, targets, eps, grad_x, grad_lower, grad_upper):
+    dev = _check(_TAIL, **{k: v for k, v in dict(grad_margin=grad_margin, targets=targets, grad_x=grad_x,
+                                                   grad_lower=grad_lower, grad_upper=grad_upper).items() if v is not None})
+    B, C = grad_margin.shape
+    _run(_margin_bwd, dev, _p(grad_margin), _p(targets), B, C, float(eps), _po(grad_x), _po(grad_lower), _po(grad_upper))
+
+
+def hinge_forward(margin, mix, loss, argmax):
+    """loss[0] = (1 - mix) * mean_b max_c relu(margin) + mix * mean relu(margin) (main.py:304-310)."""
+    dev = _check(_TAIL, margin=margin, loss=loss, argmax=argmax)
+    B, C = margin.shape
+    _run(_hinge_fwd, dev, _p(margin), B, C, float(mix), _p(loss), _p(argmax))
+
+
+def hinge_backward(margin, argmax, grad_loss, mix, grad_margin):
+    dev = _check(_TAIL, margin=margin, argmax=argmax, grad_loss=grad_loss, grad_margin=grad_margin)
+    B, C = margin.shape
+    _run(_hinge_bwd, dev, _p(margin), _p(argmax), _p(grad_loss), B, C, float(mix), _p(grad_margin))
 
 
 def _pair(v):

@@ -386,3 +386,70 @@ def bound_inf_dist(x_lower, x_upper, weight, groups=1, use_custom_cuda_func=True
     y_lower = torch.norm(-near, dim=3, p=INF, keepdim=True)
     shape = (x_lower.size(0), -1, x_lower.size(-1))
     return y_lower.view(shape), y_upper.view(shape)
+
+
+class WorstMarginF(torch.autograd.Function):
+    """Worst-case margins of the logits -x against the target class (reference: ell_inf_models.py:41-46, a dozen
+    torch primitives there): margin[b, c] = (upper[b, t_b] - lower[b, c]) / (2 eps), 0 at the target; without
+    bounds lower / upper = x -/+ eps.  One launch each way."""
+
+    @staticmethod
+    def forward(ctx, x, lower, upper, targets, eps):
+        lead = x if lower is None else lower
+        margin = torch.empty_like(lead)
+        _C.margin_forward(None if lower is not None else x, lower, upper, targets, eps, margin)
+        ctx.save_for_backward(targets)
+        ctx.eps, ctx.bounds = eps, lower is not None
+        return margin
+
+    @staticmethod
+    def backward(ctx, grad_margin):
+        targets, = ctx.saved_tensors
+        grad_margin = grad_margin.contiguous()
+        if ctx.bounds:
+            grad_lower, grad_upper = torch.empty_like(grad_margin), torch.empty_like(grad_margin)
+            _C.margin_backward(grad_margin, targets, ctx.eps, None, grad_lower, grad_upper)
+            return None, grad_lower, grad_upper, None, None
+        grad_x = torch.empty_like(grad_margin)
+        _C.margin_backward(grad_margin, targets, ctx.eps, grad_x, None, None)
+        return grad_x, None, None, None, None
+
+
+def worst_margin(x, lower, upper, targets, eps):
+    """Margins for `hinge`; the fused kernels on CUDA float32 [B, C] tensors, torch primitives otherwise."""
+    lead = x if lower is None else lower
+    if (lead.is_cuda and lead.dtype == torch.float32 and lead.dim() == 2 and eps > 0
+            and (lower is None) == (upper is None) and targets.dtype == torch.int64):
+        args = [None if t is None else t.contiguous() for t in (x, lower, upper)]
+        return WorstMarginF.apply(args[0], args[1], args[2], targets.contiguous(), float(eps))
+    if lower is None:
+        lower, upper = x - eps, x + eps
+    idx = targets.view(-1, 1)
+    return (torch.gather(upper, 1, idx) - lower).scatter(1, idx, 0) / (2 * eps)
+
+
+class HingeF(torch.autograd.Function):
+    """(1 - mix) * mean_b max_c relu(m) + mix * mean relu(m) on the margins (reference: main.py:304-310)."""
+
+    @staticmethod
+    def forward(ctx, margin, mix):
+        loss = torch.empty(1, device=margin.device, dtype=torch.float32)
+        argmax = torch.empty(margin.size(0), device=margin.device, dtype=torch.int32)
+        _C.hinge_forward(margin, mix, loss, argmax)
+        ctx.save_for_backward(margin, argmax)
+        ctx.mix = mix
+        return loss.view(())
+
+    @staticmethod
+    def backward(ctx, grad_loss):
+        margin, argmax = ctx.saved_tensors
+        grad_margin = torch.empty_like(margin)
+        _C.hinge_backward(margin, argmax, grad_loss.contiguous().view(1).float(), ctx.mix, grad_margin)
+        return grad_margin, None
+
+
+def hinge_loss(margin, mix):
+    if margin.is_cuda and margin.dtype == torch.float32 and margin.dim() == 2:
+        return HingeF.apply(margin.contiguous(), float(mix))
+    res = margin.clamp(min=0)
+    return (1 - mix) * res.max(dim=1)[0].mean() + mix * res.mean()

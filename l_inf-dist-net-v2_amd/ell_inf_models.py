@@ -8,6 +8,7 @@ import torch.nn as nn
 from core.modules import NormDist, NormDistBase
 from core.modules import BoundTanh, BoundLinear, BoundFinalLinear, BoundSequential
 from core.modules import apply_if_not_none
+from core.norm_dist import hinge_loss, worst_margin
 
 
 def check_inf_and_eval(model):
@@ -41,14 +42,12 @@ class MLPModel(nn.Module):
         x, lower, upper = self.fc_dist(paras)
         if targets is None:
             return -x * self.scalar
-        if lower is None:
-            lower = x - eps  # the network is 1-Lipschitz w.r.t. the infinity norm
-        if upper is None:
-            upper = x + eps
-        x, lower, upper = -x, -upper, -lower
-        idx = targets.view(-1, 1)
-        margin = (upper - torch.gather(lower, 1, idx)).scatter(1, idx, 0)
-        return x * self.scalar, margin / (2 * eps)
+        # logits are -x: their upper bound is -lower, the target's lower bound -upper[t]; without interval bounds the
+        # network is 1-Lipschitz w.r.t. the infinity norm: lower / upper = x -/+ eps
+        if (lower is None) != (upper is None):
+            lower = x - eps if lower is None else lower
+            upper = x + eps if upper is None else upper
+        return -x * self.scalar, worst_margin(x, lower, upper, targets, eps)
 
 
 class HybridModel(nn.Module):
@@ -80,5 +79,4 @@ class hinge:
         self.mix = mix
 
     def __call__(self, outputs, worst_outputs, targets):
-        res = worst_outputs.clamp(min=0)
-        return (1 - self.mix) * res.max(dim=1)[0].mean() + self.mix * res.mean()
+        return hinge_loss(worst_outputs, self.mix)
