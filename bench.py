@@ -236,10 +236,14 @@ def run_part(torch, _C, args, xd, wd, gd):
     gw = torch.empty_like(wd)
     _C.norm_dist_forward(xd, wd, out, 1, 8.0)
     out8 = out.clone()
+    _C.norm_dist_forward(xd, wd, out, 1, 13.7)
+    out137 = out.clone()
     _C.inf_dist_forward(xd, wd, out, pos, 1)
     calls = {
         "p8_fwd": lambda: _C.norm_dist_forward(xd, wd, out, 1, 8.0),
         "p8_bwd": lambda: _C.norm_dist_backward_input_weight(gd, xd, wd, out8, gx, gw, 1, 8.0),
+        "p13.7_fwd": lambda: _C.norm_dist_forward(xd, wd, out, 1, 13.7),
+        "p13.7_bwd": lambda: _C.norm_dist_backward_input_weight(gd, xd, wd, out137, gx, gw, 1, 13.7),
         "inf_fwd": lambda: _C.inf_dist_forward(xd, wd, out, pos, 1),
         "inf_fwd_nograd": lambda: _C.inf_dist_forward_nograd(xd, wd, out, 1),
         "inf_bwd": lambda: _C.inf_dist_backward_input_weight(gd, pos, gx, gw, 1),
@@ -270,7 +274,7 @@ def main():
     ap.add_argument("--cpu-cols", type=int, default=1024, help="output features of the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-other", action="store_true", help="skip the secondary workloads (general p, IBP, MLP, conv)")
     ap.add_argument("--part", default="all",
-                    choices=["all", "p8_fwd", "p8_bwd", "inf_fwd", "inf_fwd_nograd", "inf_bwd", "copy", "other"],
+                    choices=["all", "p8_fwd", "p8_bwd", "p13.7_fwd", "p13.7_bwd", "inf_fwd", "inf_fwd_nograd", "inf_bwd", "copy", "other"],
                     help="profiling aid: run only one entry point of the step, --steps times, on pre-allocated outputs")
     ap.add_argument("--batch", type=int, default=B, help="with --part: rows of the batch to use (e.g. 64)")
     args = ap.parse_args()

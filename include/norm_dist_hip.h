@@ -75,6 +75,13 @@ void ndist_set_skip_mode(int skip, int bounds);
  * decide (default), 0 never, 1 always the cheaper side, 2 always the rows of x, 3 always the rows of w.
  * Process-wide; initial value from NORM_DIST_HOT. */
 void ndist_set_hot_mode(int mode);
+/* Tuning and test aid, no counterpart in the reference.  For 10 < p <= 48 in the fully connected layout the forward
+ * normalises the sum by a bound of the maximum known before the reduction starts (largest |x| of the row plus
+ * largest |w|) and so needs one pass over the pairs instead of two; outputs whose sum leaves the safe float range
+ * under that bound are recomputed with their exact maximum.  mode: -1 for problems of 2e7 pairs and more (default),
+ * 0 never, 1 whenever the layout allows.  Process-wide; initial value from NORM_DIST_ROW_SCALE.  Results agree within
+ * the operator's tolerance either way. */
+void ndist_set_scaled_mode(int mode);
 /* No counterpart in the reference (PyTorch's caching allocator plays this role there).  Entry points that need
  * temporary device memory (finite-p backward, forwards whose k range is split over workgroups, the large-p paths,
  * the conv fallback) take it from arenas the library keeps per (device, stream): allocated with hipMalloc the first

@@ -60,6 +60,8 @@ _lib.ndist_set_skip_mode.argtypes = [ctypes.c_int, ctypes.c_int]
 _lib.ndist_set_skip_mode.restype = None
 _lib.ndist_set_hot_mode.argtypes = [ctypes.c_int]
 _lib.ndist_set_hot_mode.restype = None
+_lib.ndist_set_scaled_mode.argtypes = [ctypes.c_int]
+_lib.ndist_set_scaled_mode.restype = None
 _lib.ndist_release_scratch.argtypes = []
 _lib.ndist_release_scratch.restype = ctypes.c_int
 _lib.ndist_last_kernel_ms.argtypes = [ctypes.POINTER(ctypes.c_float)]
@@ -150,6 +152,12 @@ def set_hot_mode(mode=-1):
     """Tuning / test aid for the p = inf forward through hot k-tiles: -1 the device-side counts decide (default),
     0 never, 1 always the cheaper side, 2 always by the rows of x, 3 always by the rows of w."""
     _lib.ndist_set_hot_mode(int(mode))
+
+
+def set_scaled_mode(mode=-1):
+    """Tuning / test aid for the one-pass normalised forward (10 < p <= 48, fully connected layout): -1 from 2e7
+    pairs on (default), 0 never, 1 whenever the layout allows."""
+    _lib.ndist_set_scaled_mode(int(mode))
 
 
 def release_scratch():

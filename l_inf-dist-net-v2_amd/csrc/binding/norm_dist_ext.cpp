@@ -492,6 +492,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("last_kernel_ms", &last_kernel_ms);
     m.def("set_skip_mode", [](int skip, int bounds) { ndist_set_skip_mode(skip, bounds); });
     m.def("set_hot_mode", [](int mode) { ndist_set_hot_mode(mode); });
+    m.def("set_scaled_mode", [](int mode) { ndist_set_scaled_mode(mode); });
     m.def("release_scratch", &release_scratch);
     m.def("scratch_counters", &scratch_counters);
     m.def("noalloc_scratch_bytes", []() { return (long)ndist_noalloc_scratch_bytes(); });

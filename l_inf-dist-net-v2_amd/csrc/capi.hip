@@ -149,6 +149,7 @@ void ndist_set_profiling(int enable) { g_profiling.store(enable ? 1 : 0); }
 
 void ndist_set_skip_mode(int skip, int bounds) { set_skip_mode(skip, bounds); }
 void ndist_set_hot_mode(int mode) { set_hot_mode(mode); }
+void ndist_set_scaled_mode(int mode) { set_scaled_mode(mode); }
 
 int ndist_release_scratch(void) { return scratch_release_all(); }
 

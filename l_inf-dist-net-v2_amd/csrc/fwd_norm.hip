@@ -500,6 +500,113 @@ int skip_override_limit(int probed_limit) { return override_limit(g_skip_mode.lo
 int bounds_override_limit(int probed_limit) { return override_limit(g_bounds_mode.load(), probed_limit); }
 bool skip_forced_on() { return g_skip_mode.load() == 1; }
 
+// ---- one-pass normalised sum with a per-row scale (OpRowScaled) ------------------------------------------
+
+// Largest magnitude of every row of x (rows_x rows of K values) and of w (rows_w rows): one wave per row.
+__global__ __launch_bounds__(256) void row_absmax_kernel(const float* __restrict__ x, long rows_x,
+                                                         const float* __restrict__ w, long rows_w, int K, int vec,
+                                                         float* __restrict__ rx, float* __restrict__ rw) {
+    const long r = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (r >= rows_x + rows_w) return;
+    const float* __restrict__ row = r < rows_x ? x + r * K : w + (r - rows_x) * K;
+    float m = 0.f;
+    if (vec) {
+        const float4* __restrict__ v = reinterpret_cast<const float4*>(row);
+        for (int k = lane; k < K / 4; k += 64) {
+            const float4 q = v[k];
+            m = fmaxf(fmaxf(m, fmaxf(fabsf(q.x), fabsf(q.y))), fmaxf(fabsf(q.z), fabsf(q.w)));
+        }
+    } else {
+        for (int k = lane; k < K; k += 64) m = fmaxf(m, fabsf(row[k]));
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) m = fmaxf(m, __shfl_xor(m, d, 64));
+    if (lane == 0) (r < rows_x ? rx[r] : rw[r - rows_x]) = m;
+}
+
+// c[r] = p * log2(max(rx[r] + max(rw), 1e-10)): every workgroup reduces rw for itself (a few thousand values).
+__global__ __launch_bounds__(256) void row_scale_kernel(const float* __restrict__ rx, long rows_x,
+                                                        const float* __restrict__ rw, long rows_w, float p,
+                                                        float* __restrict__ c) {
+    __shared__ float part[4];
+    float m = 0.f;
+    for (long n = threadIdx.x; n < rows_w; n += 256) m = fmaxf(m, rw[n]);
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) m = fmaxf(m, __shfl_xor(m, d, 64));
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
+    const long r = (long)blockIdx.x * 256 + threadIdx.x;
+    if (r < rows_x) c[r] = p * fast_log2(fmaxf(rx[r] + m, kEps));
+}
+
+// Outputs the one-pass kernel marked with -1 (sum below the safe range, or NaN): recomputed by one wave each with
+// the exact maximum, as the two-pass operator does (maximum floored at 1e-10, its term added).  Fully connected
+// layout only (HW == 1).
+__global__ __launch_bounds__(256) void norm_fixup_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                         const Geom s, float p, float inv_p, float* __restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const long total = (long)s.M * s.COg * s.G;
+    const int CO = s.COg * s.G, K = s.CIg;
+    for (long base = ((long)blockIdx.x * 4 + (threadIdx.x >> 6)) * 64; base < total; base += (long)gridDim.x * 256) {
+        const long o = base + lane;
+        unsigned long long marked = __builtin_amdgcn_ballot_w64(o < total && out[o] < 0.f);
+        while (marked != 0) {
+            const int l = __builtin_ctzll(marked);
+            marked &= marked - 1;
+            const long oo = base + l;
+            const int b = (int)(oo / CO), cn = (int)(oo - (long)b * CO), g = cn / s.COg;
+            const float* __restrict__ xr = x + ((long)b * s.G + g) * K;
+            const float* __restrict__ wr = w + (long)cn * K;
+            float m = kEps;
+            for (int k = lane; k < K; k += 64) m = fmaxf(m, fabsf(xr[k] - wr[k]));
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) m = fmaxf(m, __shfl_xor(m, d, 64));
+            const float c = p * fast_log2(m);
+            float sum = 0.f;
+            for (int k = lane; k < K; k += 64) sum += fast_exp2(fmaf(p, fast_log2(fabsf(xr[k] - wr[k])), -c));
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) sum += __shfl_xor(sum, d, 64);
+            sum += fast_exp2(p * fast_log2(kEps) - c);
+            if (lane == 0) out[oo] = fast_exp2(fast_log2(sum) * inv_p) * m;
+        }
+    }
+}
+
+static std::atomic<int> g_scaled_mode{env_mode("NORM_DIST_ROW_SCALE")};
+void set_scaled_mode(int mode) { g_scaled_mode.store(mode < 0 ? -1 : (mode ? 1 : 0)); }
+// Up to p = 48 a scale 3.2 times the true maximum still keeps the sum above 2^-90; beyond, too many outputs would
+// take the slow exact route on ordinary data.
+constexpr float kMaxRowScaledP = 48.0f;
+static bool row_scaled_applies(const Geom& s, float p) {
+    const int mode = g_scaled_mode.load();
+    if (mode == 0 || s.HW != 1 || !(p <= kMaxRowScaledP) || skinny_applies(s)) return false;
+    return mode == 1 || (double)s.M * s.COg * s.G * s.CIg >= 2e7;
+}
+static size_t row_scaled_scratch_floats(const Geom& s) { return 2 * (size_t)s.M * s.G + (size_t)s.COg * s.G; }
+// Queues the two scale kernels, the one-pass kernel and the pass over marked outputs; `scratch` holds
+// row_scaled_scratch_floats(s) floats.  P carries the gate, if any, for the main kernel only.
+static int launch_row_scaled(FwdParams P, float* scratch, hipStream_t st) {
+    const Geom& s = P.s;
+    const long rows_x = (long)s.M * s.G, rows_w = (long)s.COg * s.G;
+    float* rx = scratch;
+    float* c = rx + rows_x;
+    float* rw = c + rows_x;
+    const int vec = s.CIg % 4 == 0 && (reinterpret_cast<uintptr_t>(P.x) & 15) == 0 && (reinterpret_cast<uintptr_t>(P.w) & 15) == 0;
+    hipLaunchKernelGGL(row_absmax_kernel, dim3((unsigned)((rows_x + rows_w + 3) / 4)), dim3(256), 0, st, P.x, rows_x, P.w,
+                       rows_w, s.CIg, vec, rx, rw);
+    hipLaunchKernelGGL(row_scale_kernel, dim3((unsigned)((rows_x + 255) / 256)), dim3(256), 0, st, rx, rows_x, rw, rows_w, P.p, c);
+    if (hip_failed(hipGetLastError())) return 4;
+    P.aux = c;
+    const int rc = launch_fwd<OpRowScaled, CfgWide4, CfgBig, CfgSmall, CfgWide>(P, st);
+    if (rc) return rc;
+    const long total = rows_x * s.COg;
+    const unsigned grid = (unsigned)std::min<long>((total + 255) / 256, 4096);
+    hipLaunchKernelGGL(norm_fixup_kernel, dim3(grid), dim3(256), 0, st, P.x, P.w, s, P.p, P.inv_p, P.out);
+    return hip_failed(hipGetLastError()) ? 4 : 0;
+}
+
 template <int IP>
 static int launch_sum(const FwdParams& P, hipStream_t st) {
     return launch_fwd<OpSum<IP>, CfgWide4, CfgBig, CfgSmall, CfgWide>(P, st);
@@ -523,11 +630,22 @@ int launch_norm_forward(const float* x, const float* w, const float* max_in, con
         // (below or above 65 % of the sampled steps) opens the gate of one of them.
         constexpr float kMinSkipP = 16.0f;  // below, the threshold 2^(-32/p) leaves almost nothing to skip
         const double pairs = (double)s.M * s.COg * s.G * s.CIg;
-        if (p < kMinSkipP || (pairs < 2e8 && !skip_forced_on()) || skinny_applies(s)) return launch_fwd<OpNormalized<false>, CfgWideT, CfgMid, CfgSmall>(P, st);
+        const bool scaled = row_scaled_applies(s, p);  // the one-pass kernel stands in for the plain two-pass one
+        if (p < kMinSkipP || (pairs < 2e8 && !skip_forced_on()) || skinny_applies(s)) {
+            float* rs = nullptr;
+            if (!scaled || scratch_alloc((void**)&rs, row_scaled_scratch_floats(s) * sizeof(float), st) != hipSuccess) {
+                (void)hipGetLastError();
+                return launch_fwd<OpNormalized<false>, CfgWideT, CfgMid, CfgSmall>(P, st);
+            }
+            int rc = launch_row_scaled(P, rs, st);
+            if (hip_failed(scratch_free(rs, st)) && !rc) rc = 4;
+            return rc;
+        }
         P.thr = exp2f(-32.0f / p);
         P.inv_thr = 1.0f / P.thr;
         float* scratch = nullptr;  // probe scratch, then the seeds of the skipping operator (values, indices)
-        if (scratch_alloc((void**)&scratch, (kProbeScratchFloats + seed_scratch_floats(s)) * sizeof(float), st) != hipSuccess) {
+        const size_t nskip = kProbeScratchFloats + seed_scratch_floats(s);
+        if (scratch_alloc((void**)&scratch, (nskip + (scaled ? row_scaled_scratch_floats(s) : 0)) * sizeof(float), st) != hipSuccess) {
             (void)hipGetLastError();  // no scratch (out of memory, or a stream under capture): the plain kernel needs none
             return launch_fwd<OpNormalized<false>, CfgWideT, CfgMid, CfgSmall>(P, st);
         }
@@ -551,7 +669,8 @@ int launch_norm_forward(const float* x, const float* w, const float* max_in, con
         }
         if (!rc) {
             P.gate_sense = 0;
-            rc = launch_fwd<OpNormalized<false>, CfgWideT, CfgMid, CfgSmall>(P, st);
+            P.aux = nullptr;
+            rc = scaled ? launch_row_scaled(P, scratch + nskip, st) : launch_fwd<OpNormalized<false>, CfgWideT, CfgMid, CfgSmall>(P, st);
         }
         if (hip_failed(scratch_free(scratch, st)) && !rc) rc = 4;
         return rc;

@@ -190,6 +190,50 @@ struct OpNormalized {
     }
 };
 
+// The normalised sum in one pass, for moderate p: any scale s >= max |x - w| gives the same result,
+// out = s * (sum (|t| / s)^p)^(1/p), as long as the sum stays inside the float range.  The scale here depends on the
+// row of x only -- its largest magnitude plus the largest magnitude in all of w, prepared as c = p * log2(s) by two
+// small kernels -- so it costs one register per row of the micro-tile, no pass for the maxima and no rescaling.
+// The scale enters the terms and the result through the same rounded c, so its rounding cancels.  An output whose
+// true maximum lies so far below the bound that the sum falls under 2^-90 (its terms near the flush-to-zero range)
+// is stored as -1; a pass over the outputs recomputes those with their exact maximum (norm_fixup_kernel).  A NaN
+// sum takes the same route.
+constexpr float kRowScaledMinSum = 8.0779357e-28f;  // 2^-90
+struct OpRowScaled {
+    static constexpr int NX = 1, PHASES = 1, NOF = 1, NOI = 0;
+    static constexpr bool PREFETCH = true;
+    static constexpr float COST = 26.8f;
+    struct Acc { float c, s; };  // c is the same for all outputs of a row: the optimiser keeps one copy per row
+    __device__ static __forceinline__ void init(Acc& a, const FwdParams& P, int kg, int m, int, int g) {
+        const int mm = m < P.s.M ? m : P.s.M - 1;
+        a.c = P.aux[(long)mm * P.s.G + g];
+        a.s = kg == 0 ? fast_exp2(P.p * fast_log2(kEps) - a.c) : 0.f;  // the reference's floor term (1e-10 / s)^p
+    }
+    template <int TN>
+    __device__ static __forceinline__ void row2(Acc (&a)[TN], const FwdParams& P, int, float x0, float,
+                                                const float (&w0)[TN], float x1, float, const float (&w1)[TN]) {
+        constexpr int N = 2 * TN;
+        float e[N];
+#pragma unroll
+        for (int j = 0; j < TN; j++) { e[j] = x0 - w0[j]; e[TN + j] = x1 - w1[j]; }
+#pragma unroll
+        for (int j = 0; j < N; j++) e[j] = fast_log2(fabsf(e[j]));
+#pragma unroll
+        for (int j = 0; j < N; j++) e[j] = fmaf(P.p, e[j], -a[j % TN].c);
+#pragma unroll
+        for (int j = 0; j < N; j++) e[j] = fast_exp2(e[j]);
+#pragma unroll
+        for (int j = 0; j < TN; j++) a[j].s += e[j];
+#pragma unroll
+        for (int j = 0; j < TN; j++) a[j].s += e[TN + j];
+    }
+    __device__ static __forceinline__ void phase_end(Acc&, const FwdParams&, int, int) {}
+    __device__ static __forceinline__ void merge(Acc& a, const Acc& b, const FwdParams&) { a.s += b.s; }
+    __device__ static __forceinline__ void finalize(const Acc& a, const FwdParams& P, float* fv, int*) {
+        fv[0] = a.s >= kRowScaledMinSum ? fast_exp2((fast_log2(a.s) + a.c) * P.inv_p) : -1.0f;
+    }
+};
+
 // The same sum for large p, in one pass and with most pairs skipped.  A pair with |t| < 2^(-32/p) * m adds less than
 // 2^-32 to a sum that is at least 1: 5120 dropped pairs change the sum by < 1.2e-6 and the result (its p-th root) by
 // that over p.  For large p almost every pair is below that threshold (p = 100: |t| < 0.80 m), so the usual work per

@@ -43,6 +43,7 @@ enum Mix {
     INF,          // d0 = x - w0 ; d1 = x - w1 ; acc = max3(acc, |d0|, |d1|)                2 pairs
     BOUND,        // t1 = w - xl ; t2 = xu - w ; lo = min3(lo, t1, t2) ; hi = max3(hi, t1, t2)   1 pair
     GENP,         // d = x - w ; e = log2|d| ; e = p*e - c ; e = exp2(e) ; acc += e           1 pair
+    GENP_BWD,     // t = x - w ; v = s*t ; e = log2|v| ; e = s*e ; e = exp2(e) ; gx += v*e ; gw += v*e   1 term
     NMIX
 };
 
@@ -69,6 +70,7 @@ static const MixInfo kMix[NMIX] = {
     {"inf: sub sub max3 (2 pairs)", 3, 2},
     {"bounds: sub sub min3 max3", 4, 1},
     {"general p: sub log fma exp add", 5, 1},
+    {"general p backward: sub mul_s log mul_s exp 2fma", 7, 1},
 };
 
 typedef float f4 __attribute__((ext_vector_type(4)));
@@ -142,6 +144,15 @@ __device__ __forceinline__ void step(float (&acc)[CH], float (&acc2)[CH], const 
         STAGE("v_exp_f32 %0, %0" : "+v"(d[c]))
         STAGE("v_add_f32 %0, %0, %1" : "+v"(acc[c]) : "v"(d[c]))
     }
+    if constexpr (MIX == GENP_BWD) {
+        STAGE("v_sub_f32 %0, %1, %2" : "=v"(d[c]) : "v"(a[c]), "v"(b[c]))
+        STAGE("v_mul_f32 %0, %1, %0" : "+v"(d[c]) : "s"(sc))
+        STAGE("v_log_f32 %0, |%1|" : "=v"(e[c]) : "v"(d[c]))
+        STAGE("v_mul_f32 %0, %1, %0" : "+v"(e[c]) : "s"(sc))
+        STAGE("v_exp_f32 %0, %0" : "+v"(e[c]))
+        STAGE("v_fma_f32 %0, %1, %2, %0" : "+v"(acc[c]) : "v"(d[c]), "v"(e[c]))
+        STAGE("v_fma_f32 %0, %1, %2, %0" : "+v"(acc2[c]) : "v"(d[c]), "v"(e[c]))
+    }
 #undef STAGE
     (void)f;
 }
@@ -182,7 +193,7 @@ static int g_cus = 256;
 
 template <int MIX, int CH, int NOPS = 0>
 void run_case(int waves) {
-    constexpr int NI_RAW = MIX == P8_FWD ? 4 : (MIX == P8_BWD || MIX == P8_BWD_V || MIX == P8_BWD_LDS) ? 7 : MIX == INF ? 3 : MIX == BOUND ? 4 : MIX == GENP ? 5 : 1;
+    constexpr int NI_RAW = MIX == P8_FWD ? 4 : (MIX == P8_BWD || MIX == P8_BWD_V || MIX == P8_BWD_LDS) ? 7 : MIX == INF ? 3 : MIX == BOUND ? 4 : MIX == GENP ? 5 : MIX == GENP_BWD ? 7 : 1;
     constexpr int UNROLL = (128 / (CH * NI_RAW)) > 0 ? (128 / (CH * NI_RAW)) : 1;
     auto kern = mix_kernel<MIX, CH, UNROLL, NOPS>;
     const int blocks = g_cus * waves;

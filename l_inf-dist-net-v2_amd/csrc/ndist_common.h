@@ -250,6 +250,9 @@ int skip_override_limit(int probed_limit);
 bool skip_forced_on();
 int bounds_override_limit(int probed_limit);
 void set_skip_mode(int skip, int bounds);
+// Tuning and test aid (ndist_set_scaled_mode / NORM_DIST_ROW_SCALE): the one-pass normalised forward for
+// 10 < p <= 48 in the fully connected layout; -1 from 2e7 pairs on (default), 0 never, 1 whenever the layout allows.
+void set_scaled_mode(int mode);
 int launch_unfold(const float* x, const UnfoldGeom& u, float* out, hipStream_t st);
 int launch_fold(const float* gout, const UnfoldGeom& u, float* gx, hipStream_t st);
 // the patches as rows [B * OH * OW][C * kh * kw] (the transpose of the unfolded tensor); -1: geometry not served
