@@ -75,42 +75,104 @@ __global__ __launch_bounds__(256) void scatter_atomic_kernel(const float* __rest
     }
 }
 
+// LDS float add of one value per lane, with the lanes of a wave that target the same word combined first.  Codes
+// cluster: every output of a batch row whose largest |x| dominates names the same input, every batch row of an
+// output whose weight row has one dominant entry names the same weight, and thousands of adds to one LDS word
+// serialise.  At most two clusters of eight or more lanes are summed across the wave (butterfly) and added once by
+// their first lane; what remains goes through plain adds.  off < 0: the lane has nothing to add.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+    return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+// Sum over the 64 lanes of a wave (all active), the same value in every lane: butterfly inside the quads
+// (quad_perm [1,0,3,2], [2,3,0,1]), rotations by 4 and 8 inside the rows of 16, then the four row sums.
+__device__ __forceinline__ float wave_sum(float v) {
+    v = dpp_add<0xB1>(v);
+    v = dpp_add<0x4E>(v);
+    v = dpp_add<0x124>(v);
+    v = dpp_add<0x128>(v);
+    const int i = __builtin_bit_cast(int, v);
+    return (__builtin_bit_cast(float, __builtin_amdgcn_readlane(i, 0)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(i, 16))) +
+           (__builtin_bit_cast(float, __builtin_amdgcn_readlane(i, 32)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(i, 48)));
+}
+__device__ __forceinline__ void lds_add_clustered(float* base, int off, float v) {
+    const int lane = threadIdx.x & 63;
+    bool active = off >= 0;
+#pragma unroll 1
+    for (int round = 0; round < 2; round++) {
+        const unsigned long long todo = __builtin_amdgcn_ballot_w64(active);
+        if (todo == 0) return;
+        const int leader = __builtin_ctzll(todo);
+        const int loff = __builtin_amdgcn_readlane(off, leader);
+        const bool mine = active && off == loff;
+        const unsigned long long grp = __builtin_amdgcn_ballot_w64(mine);
+        if (__builtin_popcountll(grp) < 8) break;
+        const float sum = wave_sum(mine ? v : 0.f);
+        if (lane == leader) atomicAdd(base + loff, sum);
+        active = active && !mine;
+    }
+    if (active) atomicAdd(base + off, v);
+}
+
+constexpr int kScatterBatch = 8;  // outputs whose codes and gradients a thread requests before it adds any of them
+
 // ---- privatised path, HW == 1 ---------------------------------------------------------------------------
 // grad_input: one workgroup per (b, g); LDS holds the CIg-long row (two rows for the interval variant).
 template <bool BOUND>
-__global__ __launch_bounds__(256) void scatter_gx_rows_kernel(const float* __restrict__ g1, const float* __restrict__ g2,
+__global__ __launch_bounds__(1024) void scatter_gx_rows_kernel(const float* __restrict__ g1, const float* __restrict__ g2,
                                                               const int32_t* __restrict__ p1,
                                                               const int32_t* __restrict__ p2, float* __restrict__ gx1,
                                                               float* __restrict__ gx2, const Geom s) {
     extern __shared__ float row[];  // [BOUND ? 2 : 1][CIg]
-    const int b = blockIdx.x, g = blockIdx.y;
+    const int b = blockIdx.x, g = blockIdx.y, nt = blockDim.x;
     const int nrow = (BOUND ? 2 : 1) * s.CIg;
     const long xbase = x_off(s, b, g, 0, 0);
     // 16-byte LDS and global accesses when the rows allow it (the dynamic LDS base is 16-byte aligned)
     const bool vec = s.CIg % 4 == 0 && (uintptr_t)(gx1 + xbase) % 16 == 0 && (!BOUND || (uintptr_t)(gx2 + xbase) % 16 == 0);
     if (vec) {
-        for (int i = threadIdx.x; i < nrow / 4; i += 256) reinterpret_cast<float4*>(row)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int i = threadIdx.x; i < nrow / 4; i += nt) reinterpret_cast<float4*>(row)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
     } else {
-        for (int i = threadIdx.x; i < nrow; i += 256) row[i] = 0.f;
+        for (int i = threadIdx.x; i < nrow; i += nt) row[i] = 0.f;
     }
     __syncthreads();
     const long obase = y_off(s, b, g, 0, 0);
-    for (int co = threadIdx.x; co < s.COg; co += 256) {
-        const Route a = BOUND ? route_lower(p1[obase + co], g1[obase + co]) : route_inf(p1[obase + co], g1[obase + co]);
-        if (a.target >= 0 && a.idx < s.CIg) atomicAdd(row + a.target * s.CIg + a.idx, a.v);
-        if (BOUND) {
-            const Route c = route_upper(p2[obase + co], g2[obase + co]);
-            if (c.idx < s.CIg) atomicAdd(row + c.target * s.CIg + c.idx, c.v);
+    // the loads of kScatterBatch outputs are issued together: one memory latency per batch, not per output
+    // (the loop bounds are the same for all threads: lds_add_clustered needs whole waves)
+    for (int k0 = 0; k0 < s.COg; k0 += nt * kScatterBatch) {
+        const int c0 = k0 + threadIdx.x;
+        int32_t pa[kScatterBatch], pb[kScatterBatch];
+        float ga[kScatterBatch], gb[kScatterBatch];
+#pragma unroll
+        for (int u = 0; u < kScatterBatch; u++) {
+            const int co = min(c0 + u * nt, s.COg - 1);  // clamped, not guarded: no branch between the loads
+            pa[u] = p1[obase + co];
+            ga[u] = g1[obase + co];
+            if (BOUND) {
+                pb[u] = p2[obase + co];
+                gb[u] = g2[obase + co];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kScatterBatch; u++) {
+            if (k0 + u * nt < s.COg) {  // some thread of this step has an output
+                const bool live = c0 + u * nt < s.COg;
+                const Route a = BOUND ? route_lower(pa[u], ga[u]) : route_inf(pa[u], ga[u]);
+                lds_add_clustered(row, live && a.target >= 0 && a.idx < s.CIg ? a.target * s.CIg + a.idx : -1, a.v);
+                if (BOUND) {
+                    const Route c = route_upper(pb[u], gb[u]);
+                    lds_add_clustered(row, live && c.idx < s.CIg ? c.target * s.CIg + c.idx : -1, c.v);
+                }
+            }
         }
     }
     __syncthreads();
     if (vec) {
-        for (int i = threadIdx.x; i < s.CIg / 4; i += 256) {
+        for (int i = threadIdx.x; i < s.CIg / 4; i += nt) {
             reinterpret_cast<float4*>(gx1 + xbase)[i] = reinterpret_cast<const float4*>(row)[i];
             if (BOUND) reinterpret_cast<float4*>(gx2 + xbase)[i] = reinterpret_cast<const float4*>(row + s.CIg)[i];
         }
     } else {
-        for (int i = threadIdx.x; i < s.CIg; i += 256) {
+        for (int i = threadIdx.x; i < s.CIg; i += nt) {
             gx1[xbase + i] = row[i];
             if (BOUND) gx2[xbase + i] = row[s.CIg + i];
         }
@@ -124,7 +186,19 @@ __global__ __launch_bounds__(256) void scatter_gw_rows_kernel(const float* __res
                                                               const int32_t* __restrict__ p2, float* __restrict__ gw,
                                                               const Geom s, int R) {
     extern __shared__ float rows[];  // [R][CIg]
-    const int g = blockIdx.y, co0 = blockIdx.x * R;
+    // Workgroups are handed to the eight XCDs in turn, and a workgroup uses 4 R bytes of every 128-byte line of
+    // grad_output and codes it touches: numbered as launched, the neighbours that share its lines would sit on
+    // the other seven XCDs and every L2 would fetch every line.  Renumbered so that each XCD owns a contiguous
+    // range of co blocks, the workgroups resident on one XCD share the lines.
+    int g, cb;
+    {
+        const int total = gridDim.x * gridDim.y, id = blockIdx.y * gridDim.x + blockIdx.x;
+        const int q = total / 8, rem = total % 8, xcd = id % 8, slot = id / 8;
+        const int logical = xcd * q + min(xcd, rem) + slot;
+        g = logical / gridDim.x;
+        cb = logical - g * gridDim.x;
+    }
+    const int co0 = cb * R;
     const int nr = min(R, s.COg - co0);
     float* dst = gw + w_off(s, g, co0, 0);
     const bool vec = s.CIg % 4 == 0 && (uintptr_t)dst % 16 == 0;
@@ -135,14 +209,17 @@ __global__ __launch_bounds__(256) void scatter_gw_rows_kernel(const float* __res
     }
     __syncthreads();
     // thread -> (b, r): r fastest so that one b's R codes are read as one contiguous segment
-    for (int i = threadIdx.x; i < s.B * nr; i += 256) {
-        const int b = i / nr, r = i - b * nr;
+    const int n = s.B * nr;
+    for (int i0 = 0; i0 < n; i0 += 256) {
+        const int i = i0 + threadIdx.x;
+        const bool live = i < n;
+        const int b = live ? i / nr : 0, r = live ? i - b * nr : 0;
         const long o = y_off(s, b, g, co0 + r, 0);
         const Route a = BOUND ? route_lower(p1[o], g1[o]) : route_inf(p1[o], g1[o]);
-        if (a.target >= 0 && a.idx < s.CIg) atomicAdd(rows + r * s.CIg + a.idx, -a.v);
+        lds_add_clustered(rows, live && a.target >= 0 && a.idx < s.CIg ? r * s.CIg + a.idx : -1, -a.v);
         if (BOUND) {
             const Route c = route_upper(p2[o], g2[o]);
-            if (c.idx < s.CIg) atomicAdd(rows + r * s.CIg + c.idx, -c.v);
+            lds_add_clustered(rows, live && c.idx < s.CIg ? r * s.CIg + c.idx : -1, -c.v);
         }
     }
     __syncthreads();
@@ -392,12 +469,17 @@ static int scatter_backward(const float* g1, const float* g2, const int32_t* p1,
         NDIST_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&scatter_gw_rows_kernel<BOUND>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, kScatterLdsBudget));
         KernelTimer timer(st);  // both row kernels together
-        hipLaunchKernelGGL(scatter_gx_rows_kernel<BOUND>, dim3(s.B, s.G), dim3(256), gx_lds, st, g1, g2, p1, p2, gx1, gx2,
-                           s);
+        // a row of 2048 outputs and more gets 1024 threads: the kernel has one workgroup per batch row and lives on
+        // how many loads each of them keeps in flight
+        hipLaunchKernelGGL(scatter_gx_rows_kernel<BOUND>, dim3(s.B, s.G), dim3(s.COg >= 2048 ? 1024 : 256), gx_lds, st, g1, g2,
+                           p1, p2, gx1, gx2, s);
         if (hip_failed(hipGetLastError())) return 4;
         if (gw) {
             int R = (int)((size_t)kScatterLdsBudget / ((size_t)s.CIg * sizeof(float)));
-            R = R > 4 ? 4 : R;  // R >= 1 because one row fits the budget
+            // R >= 1 because one row fits the budget.  Two rows: with the XCD-aware numbering the L2 makes up for the
+            // short segments, and four workgroups of 2 x 20 KB per compute unit overlap their fill, scatter and
+            // store phases better than two of 4 x 20 KB (31.7 against 36.5 us at 512 x 5120 x 5120)
+            R = R > 2 ? 2 : R;
             hipLaunchKernelGGL(scatter_gw_rows_kernel<BOUND>, dim3(ceil_div(s.COg, R), s.G), dim3(256),
                                (size_t)R * s.CIg * sizeof(float), st, g1, g2, p1, p2, gw, s, R);
             if (hip_failed(hipGetLastError())) return 4;
