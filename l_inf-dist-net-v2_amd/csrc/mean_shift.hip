@@ -1,5 +1,5 @@
-// Mean shift and bias of a distance layer in two or three launches: what follows every operator call in the
-// reference's layers (core/modules/norm_dist.py:35-38 -> core/modules/basic_modules.py:121-132): the per-channel
+// Mean shift and bias of a distance layer in one launch (fully connected layout, shift_fused_kernel) or two to
+// three: what follows every operator call in the reference's layers (core/modules/norm_dist.py:35-38 -> core/modules/basic_modules.py:121-132): the per-channel
 // batch mean of x (training; the running mean in evaluation) is subtracted from x and from both interval bounds, the
 // moving average is updated, and the layer's bias is added.  With torch primitives this is a reduction, an in-place
 // update and an elementwise kernel per tensor; here:
@@ -98,6 +98,82 @@ __global__ __launch_bounds__(256) void shift_apply_kernel(const float* __restric
 
 static bool aligned16(const void* p) { return p == nullptr || (uintptr_t)p % 16 == 0; }
 
+// All three steps in one launch for the fully connected layout (HW == 1, C % 4 == 0): a workgroup owns 32 channels
+// (one 128-byte line per batch row), adds its rows up in a fixed order (thread (r, q) the rows r, r + 32, ... of
+// four channels, then the 32 partial sums in order), writes mean / column sum / moving average and goes over its
+// rows a second time to subtract (that pass finds them in the L2).  t2 and t3 only join the sum (the adjoint: the
+// gradients of the two bounds).
+constexpr int kFusedCols = 32;
+__global__ __launch_bounds__(256) void shift_fused_kernel(const float* __restrict__ t1, const float* __restrict__ t2,
+                                                          const float* __restrict__ t3, float* __restrict__ y1, int B, int C,
+                                                          float inv_count, float momentum, float* __restrict__ running_mean,
+                                                          float* __restrict__ mean_out, float* __restrict__ colsum_out,
+                                                          const float* __restrict__ bias1, const float* __restrict__ bias2) {
+    __shared__ float4 part[32][8];
+    const int q = threadIdx.x & 7, r = threadIdx.x >> 3;
+    const int c = blockIdx.x * kFusedCols + q * 4;
+    const bool live = c < C;
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (live) {
+#pragma unroll 4
+        for (int b = r; b < B; b += 32) {
+            float4 v = *reinterpret_cast<const float4*>(t1 + (long)b * C + c);
+            if (t2 != nullptr) {
+                const float4 u = *reinterpret_cast<const float4*>(t2 + (long)b * C + c);
+                v = make_float4(v.x + u.x, v.y + u.y, v.z + u.z, v.w + u.w);
+            }
+            if (t3 != nullptr) {
+                const float4 u = *reinterpret_cast<const float4*>(t3 + (long)b * C + c);
+                v = make_float4(v.x + u.x, v.y + u.y, v.z + u.z, v.w + u.w);
+            }
+            s = make_float4(s.x + v.x, s.y + v.y, s.z + v.z, s.w + v.w);
+        }
+    }
+    part[r][q] = s;
+    __syncthreads();
+    float4 tot = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int i = 0; i < 32; i++) {
+        const float4 v = part[i][q];
+        tot = make_float4(tot.x + v.x, tot.y + v.y, tot.z + v.z, tot.w + v.w);
+    }
+    if (!live) return;
+    const float4 mean = make_float4(tot.x * inv_count, tot.y * inv_count, tot.z * inv_count, tot.w * inv_count);
+    if (r == 0) {
+        if (mean_out != nullptr) *reinterpret_cast<float4*>(mean_out + c) = mean;
+        if (colsum_out != nullptr) *reinterpret_cast<float4*>(colsum_out + c) = tot;
+        if (running_mean != nullptr) {
+            const float k = 1.0f - momentum;
+            running_mean[c] = running_mean[c] * k + mean.x * momentum;
+            running_mean[c + 1] = running_mean[c + 1] * k + mean.y * momentum;
+            running_mean[c + 2] = running_mean[c + 2] * k + mean.z * momentum;
+            running_mean[c + 3] = running_mean[c + 3] * k + mean.w * momentum;
+        }
+    }
+    if (y1 == nullptr) return;
+    float4 sft = mean;
+    if (bias1 != nullptr) sft = make_float4(sft.x - bias1[c], sft.y - bias1[c + 1], sft.z - bias1[c + 2], sft.w - bias1[c + 3]);
+    if (bias2 != nullptr) sft = make_float4(sft.x - bias2[c], sft.y - bias2[c + 1], sft.z - bias2[c + 2], sft.w - bias2[c + 3]);
+#pragma unroll 4
+    for (int b = r; b < B; b += 32) {
+        const float4 v = *reinterpret_cast<const float4*>(t1 + (long)b * C + c);
+        *reinterpret_cast<float4*>(y1 + (long)b * C + c) = make_float4(v.x - sft.x, v.y - sft.y, v.z - sft.z, v.w - sft.w);
+    }
+}
+
+static bool fused_applies(const float* t1, const float* t2, const float* t3, const float* y1, const float* m1, const float* m2,
+                          int C, int HW) {
+    return HW == 1 && C % 4 == 0 && aligned16(t1) && aligned16(t2) && aligned16(t3) && aligned16(y1) && aligned16(m1) &&
+           aligned16(m2);
+}
+static int launch_fused(const float* t1, const float* t2, const float* t3, float* y1, int B, int C, float momentum,
+                        float* running_mean, float* mean_out, float* colsum_out, const float* b1, const float* b2,
+                        hipStream_t st) {
+    hipLaunchKernelGGL(shift_fused_kernel, dim3(ceil_div(C, kFusedCols)), dim3(256), 0, st, t1, t2, t3, y1, B, C,
+                       1.0f / (float)B, momentum, running_mean, mean_out, colsum_out, b1, b2);
+    return hip_failed(hipGetLastError()) ? 4 : 0;
+}
+
 static int launch_apply(const float* t1, const float* t2, const float* t3, float* y1, float* y2, float* y3,
                         const float* mean, const float* b1, const float* b2, int B, int C, int HW, hipStream_t st) {
     const long total = (long)B * C * HW;
@@ -149,6 +225,8 @@ int ndist_mean_shift_forward(const float* x, const float* lower, const float* up
     if (training) {
         // the batch mean of x (the reference requires x in training, core/modules/basic_modules.py:123)
         if (x == nullptr || mean_out == nullptr) return NDIST_ERR_NULL_POINTER;
+        if (lower == nullptr && upper == nullptr && fused_applies(x, nullptr, nullptr, y, mean_out, nullptr, C, HW))
+            return launch_fused(x, nullptr, nullptr, y, B, C, momentum, running_mean, mean_out, nullptr, bias1, bias2, st);
         if (int rc = launch_colmean(x, nullptr, nullptr, B, C, HW, momentum, running_mean, mean_out, nullptr, st)) return rc;
         mean = mean_out;
     }  // evaluation without a running mean: biases only
@@ -173,6 +251,9 @@ int ndist_mean_shift_backward(const float* grad_y, const float* grad_y_lower, co
     hipStream_t st = (hipStream_t)stream;
     if (!training && colsum_out == nullptr) return NDIST_OK;  // evaluation: grad_x is grad_y itself, nothing to do
     if (mean_scratch == nullptr) return NDIST_ERR_NULL_POINTER;
+    if (training && grad_x != nullptr && lead == grad_y &&
+        fused_applies(lead, rest[0], rest[1], grad_x, mean_scratch, colsum_out, C, HW))
+        return launch_fused(lead, rest[0], rest[1], grad_x, B, C, 0.f, nullptr, mean_scratch, colsum_out, nullptr, nullptr, st);
     if (int rc = launch_colmean(lead, rest[0], rest[1], B, C, HW, 0.f, nullptr, mean_scratch, colsum_out, st)) return rc;
     if (!training || grad_x == nullptr) return NDIST_OK;
     if (grad_y == nullptr) {
