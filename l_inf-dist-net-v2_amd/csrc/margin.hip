@@ -18,7 +18,12 @@ __global__ __launch_bounds__(256) void margin_forward_kernel(const float* __rest
     const long i = (long)blockIdx.x * 256 + threadIdx.x;
     if (i >= (long)B * C) return;
     const int b = (int)(i / C), c = (int)(i - (long)b * C);
-    const int t = (int)targets[b];
+    const long long tl = targets[b];
+    if (tl < 0 || tl >= C) {  // a label outside the classes must not become a wild read: the row comes out as NaN
+        margin[i] = __builtin_nanf("");
+        return;
+    }
+    const int t = (int)tl;
     const float up_t = upper != nullptr ? upper[(long)b * C + t] : x[(long)b * C + t] + eps;
     const float lo_c = lower != nullptr ? lower[i] : x[i] - eps;
     margin[i] = c == t ? 0.f : (up_t - lo_c) / (2.0f * eps);
@@ -33,7 +38,8 @@ __global__ __launch_bounds__(256) void margin_backward_kernel(const float* __res
                                                               float* __restrict__ grad_upper) {
     const int b = blockIdx.x * 256 + threadIdx.x;
     if (b >= B) return;
-    const int t = (int)targets[b];
+    const long long tl = targets[b];
+    const int t = tl < 0 || tl >= C ? -1 : (int)tl;  // a label outside the classes: no target column to write
     const float inv = 1.0f / (2.0f * eps);
     float sum = 0.f;
     for (int c = 0; c < C; c++) {
@@ -43,6 +49,7 @@ __global__ __launch_bounds__(256) void margin_backward_kernel(const float* __res
         if (grad_lower != nullptr) grad_lower[(long)b * C + c] = -v;
         if (grad_upper != nullptr) grad_upper[(long)b * C + c] = 0.f;
     }
+    if (t < 0) return;
     if (grad_x != nullptr) grad_x[(long)b * C + t] = sum;
     if (grad_upper != nullptr) grad_upper[(long)b * C + t] = sum;
 }

@@ -67,3 +67,16 @@ def test_model_tail_matches_torch_primitives():
     assert abs(loss.item() - l.item()) <= 1e-5 * abs(l.item()) + 1e-7
     loss.backward()
     assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in model.parameters())
+
+
+def test_label_outside_the_classes_gives_nan_rows_not_a_fault():
+    from core import _C
+    x = torch.randn(6, 10, device="cuda")
+    t = torch.tensor([0, 9, 10, -1, 3, 4], device="cuda")
+    m = torch.empty_like(x)
+    _C.margin_forward(x, None, None, t, 0.1, m)
+    bad = torch.isnan(m).all(dim=1).cpu()
+    assert bad.tolist() == [False, False, True, True, False, False]
+    gx = torch.full_like(x, 7.0)
+    _C.margin_backward(torch.ones_like(x), t, 0.1, gx, None, None)
+    assert torch.isfinite(gx).all()

@@ -54,6 +54,25 @@ def test_argument_validation_returns_status_without_touching_a_device():
     assert g(dummy, dummy, 2, 4, 4, 1, 1, dummy, float("inf"), None) == 3
 
 
+def test_tail_entry_points_validate_their_arguments():
+    from core import _C
+    lib = ctypes.CDLL(_C.LIBRARY_PATH)
+    dummy = ctypes.c_void_p(16)
+    m = lib.ndist_margin_forward
+    m.restype = ctypes.c_int
+    m.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 2 + [ctypes.c_float] + [ctypes.c_void_p] * 2
+    assert m(None, None, None, dummy, 4, 10, 0.1, dummy, None) == 1       # neither x nor both bounds
+    assert m(None, dummy, None, dummy, 4, 10, 0.1, dummy, None) == 1      # one bound alone
+    assert m(dummy, None, None, None, 4, 10, 0.1, dummy, None) == 1       # no targets
+    assert m(dummy, None, None, dummy, 0, 10, 0.1, dummy, None) == 2      # empty batch
+    assert m(dummy, None, None, dummy, 4, 10, 0.0, dummy, None) == 2      # the margin divides by 2 eps
+    h = lib.ndist_hinge_forward
+    h.restype = ctypes.c_int
+    h.argtypes = [ctypes.c_void_p] + [ctypes.c_int] * 2 + [ctypes.c_float] + [ctypes.c_void_p] * 3
+    assert h(None, 4, 10, 0.25, dummy, dummy, None) == 1
+    assert h(dummy, 4, 0, 0.25, dummy, dummy, None) == 2
+
+
 def test_binding_rejects_cpu_and_non_contiguous_tensors():
     from core import _C
     x = torch.zeros(2, 4, 1)
