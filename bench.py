@@ -182,6 +182,8 @@ def other_workloads(torch, _C, xd, wd, gd):
 
     set_p(8.0)
     res["mlp_6x5120_b512_p8_train_step"] = tm(train_step)
+    set_p(13.7)  # early in the exponent's ramp: exp2 / log2 kernels, nothing to skip yet
+    res["mlp_6x5120_b512_p13.7_train_step"] = tm(train_step)
     set_p(100.0)  # mid-schedule exponent: general-p kernels, pair skipping where the probe allows it
     res["mlp_6x5120_b512_p100_train_step"] = tm(train_step)
     set_p(float("inf"))

@@ -191,6 +191,24 @@ int ndist_inf_and_bound_forward(const float* input, const float* inputL, const f
                                 int CO, int CI, int G, int HW, float* output, int32_t* pos, float* outputL,
                                 float* outputU, int32_t* posL, int32_t* posU, ndist_stream_t stream);
 
+/* ---- evaluation with the weights' pre-pass kept between calls ---------------------------------------------------
+ * No counterpart in the reference.  On large fully connected problems the p = inf forwards start with a pass over the
+ * weights (largest magnitude, its position and the 32-wide tile maxima of every row: it reads all of w).  While the
+ * weights do not change -- evaluation, certification, serving -- that pass can be done once:
+ *   ndist_weight_cache_bytes      size of the caller-allocated device buffer for a [CO, CI / G] weight (0: bad shape)
+ *   ndist_weight_cache_prepare    fills it from `weight` (one kernel)
+ *   ..._nograd_cached             ndist_inf_dist_forward_nograd / ndist_inf_and_bound_forward_nograd reading the pass
+ *                                 from `cache` instead of redoing it; results are bit-identical.
+ * The cache is only valid for the weight values it was prepared from: prepare it again after every change of the
+ * weights (the library cannot check).  Problems that use no pre-pass (small ones, the conv layout) ignore it. */
+long long ndist_weight_cache_bytes(int CO, int CI, int G);
+int ndist_weight_cache_prepare(const float* weight, int CO, int CI, int G, void* cache, ndist_stream_t stream);
+int ndist_inf_dist_forward_nograd_cached(const float* input, const float* weight, const void* cache, int B, int CO, int CI,
+                                         int G, int HW, float* output, ndist_stream_t stream);
+int ndist_inf_and_bound_forward_nograd_cached(const float* input, const float* inputL, const float* inputU,
+                                              const float* weight, const void* cache, int B, int CO, int CI, int G, int HW,
+                                              float* output, float* outputL, float* outputU, ndist_stream_t stream);
+
 /* ---- mean shift and bias of a distance layer ------------------------------------------------------------------
  * The reference has no kernel of its own here: every layer follows the operator with MeanShift and a bias add
  * written in torch primitives (core/modules/norm_dist.py:35-38, core/modules/basic_modules.py:121-132).  These two

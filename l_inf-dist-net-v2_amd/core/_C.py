@@ -88,6 +88,11 @@ _bnd_bwd_xw = _sig("ndist_bound_inf_dist_backward_input_weight", _P, _P, _P, _P,
 _joint_ng = _sig("ndist_inf_and_bound_forward_nograd", _P, _P, _P, _P, *_DIMS, _P, _P, _P, _P)
 _joint = _sig("ndist_inf_and_bound_forward", _P, _P, _P, _P, *_DIMS, _P, _P, _P, _P, _P, _P, _P)
 _ms_fwd = _sig("ndist_mean_shift_forward", _P, _P, _P, _I, _I, _I, _I, _F, _P, _P, _P, _P, _P, _P, _P, _P)
+_lib.ndist_weight_cache_bytes.argtypes = [_I, _I, _I]
+_lib.ndist_weight_cache_bytes.restype = ctypes.c_longlong
+_wcache_prepare = _sig("ndist_weight_cache_prepare", _P, _I, _I, _I, _P, _P)
+_inf_ng_cached = _sig("ndist_inf_dist_forward_nograd_cached", _P, _P, _P, _I, _I, _I, _I, _I, _P, _P)
+_joint_ng_cached = _sig("ndist_inf_and_bound_forward_nograd_cached", _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P)
 _margin_fwd = _sig("ndist_margin_forward", _P, _P, _P, _P, _I, _I, _F, _P, _P)
 _margin_bwd = _sig("ndist_margin_backward", _P, _P, _I, _I, _F, _P, _P, _P, _P)
 _hinge_fwd = _sig("ndist_hinge_forward", _P, _I, _I, _F, _P, _P, _P)
@@ -358,6 +363,34 @@ def inf_and_bound_forward_nograd(input, inputL, inputU, weight, output, outputL,
     B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
     _run(_joint_ng, dev, _p(input), _p(inputL), _p(inputU), _p(weight), B, CO, CI, G, HW, _p(output), _p(outputL),
          _p(outputU))
+
+
+def weight_cache(weight, G):
+    """The p = inf forwards' pre-pass over the weights (row maxima, their positions, 32-wide tile maxima) as a device
+    buffer to pass to the *_cached forwards while the weights stay as they are: evaluation, certification, serving.
+    (No counterpart in the reference; ctypes on either binding.)"""
+    dev = _check({}, weight=weight)
+    CO, CIg = weight.shape
+    nbytes = _lib.ndist_weight_cache_bytes(CO, CIg * G, G)
+    if nbytes <= 0:
+        raise NormDistError("ndist_weight_cache_bytes: bad shape", 2)
+    cache = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=weight.device)
+    _run(_wcache_prepare, dev, _p(weight), CO, CIg * G, G, _p(cache))
+    return cache
+
+
+def inf_dist_forward_nograd_cached(input, weight, cache, output, G):
+    dev = _check({}, input=input, weight=weight, cache=cache, output=output)
+    B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
+    _run(_inf_ng_cached, dev, _p(input), _p(weight), _p(cache), B, CO, CI, G, HW, _p(output))
+
+
+def inf_and_bound_forward_nograd_cached(input, inputL, inputU, weight, cache, output, outputL, outputU, G):
+    dev = _check({}, input=input, inputL=inputL, inputU=inputU, weight=weight, cache=cache, output=output,
+                 outputL=outputL, outputU=outputU)
+    B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
+    _run(_joint_ng_cached, dev, _p(input), _p(inputL), _p(inputU), _p(weight), _p(cache), B, CO, CI, G, HW, _p(output),
+         _p(outputL), _p(outputU))
 
 
 def inf_and_bound_forward(input, inputL, inputU, weight, output, pos, outputL, outputU, posL, posU, G):

@@ -8,7 +8,7 @@ import torch
 import torch.nn as nn
 
 from core.norm_dist import (norm_dist, bound_inf_dist, conv_norm_dist, conv_bound_inf_dist, mean_shift_bias,
-                            inf_dist_with_bounds)
+                            inf_dist_with_bounds, inf_dist_nograd, WeightCache)
 from .basic_modules import MeanShift, apply_if_not_none
 
 
@@ -27,14 +27,21 @@ class NormDistBase(nn.Module):
         self.bias = nn.Parameter(torch.zeros(out_features)) if bias else None
         NormDistBase.tag = getattr(NormDistBase, 'tag', 0) + 1
         self.tag = NormDistBase.tag
+        self._weight_cache = WeightCache()  # plain attribute: not a parameter or buffer, never in the state dict
 
     def forward(self, x=None, lower=None, upper=None):
+        # evaluation without gradients: the weights stand still from call to call, their pre-pass is kept
+        frozen = not self.training and not torch.is_grad_enabled() and math.isinf(self.p) and self.weight.is_cuda
+        cache = self._weight_cache if frozen else None
         if x is not None and lower is not None and upper is not None and math.isinf(self.p) and x.is_cuda:
             # the distance and its bounds against the same weights: one call (shares the pre-pass over the weights)
-            x, lower, upper = inf_dist_with_bounds(x, lower, upper, self.weight, self.groups, tag=self.tag)
+            x, lower, upper = inf_dist_with_bounds(x, lower, upper, self.weight, self.groups, tag=self.tag, cache=cache)
             return self._shift_and_bias(x, lower, upper)
         if x is not None:
-            x = norm_dist(x, self.weight, self.p, self.groups, tag=self.tag)
+            if cache is not None and x.is_cuda and x.dtype == torch.float32:
+                x = inf_dist_nograd(x, self.weight, self.groups, cache=cache)
+            else:
+                x = norm_dist(x, self.weight, self.p, self.groups, tag=self.tag)
         if lower is not None and upper is not None:
             assert math.isinf(self.p)  # interval propagation exists for the infinity distance only
             lower, upper = bound_inf_dist(lower, upper, self.weight, self.groups, tag=self.tag)

@@ -288,7 +288,36 @@ def conv_bound_inf_dist(x_lower, x_upper, weight, kernel_size, dilation=1, paddi
                           unfold(x_upper, kernel_size, dilation, padding, stride), weight, groups, tag=tag)
 
 
-def inf_dist_with_bounds(x, x_lower, x_upper, weight, groups=1, tag=None):
+class WeightCache:
+    """The p = inf forwards' pre-pass over a layer's weights, kept while the weights stay as they are (evaluation,
+    certification, serving) and redone when they change: the key is the parameter's storage address and version
+    counter, which every in-place update (optimizer step, load_state_dict, copy_) advances.  No counterpart in the
+    reference."""
+
+    def __init__(self):
+        self._key, self._buffer = None, None
+
+    def get(self, weight, groups):
+        key = (weight.data_ptr(), weight._version, tuple(weight.shape), groups, weight.device)
+        if key != self._key:
+            self._buffer = _C.weight_cache(weight.detach().contiguous(), groups)
+            self._key = key
+        return self._buffer
+
+
+def inf_dist_nograd(x, weight, groups=1, cache=None):
+    """The infinity distance without gradients, optionally with the weights' pre-pass taken from `cache`
+    (WeightCache)."""
+    x, weight = x.contiguous(), weight.contiguous()
+    y = _new_output(x, weight)
+    if cache is not None:
+        _C.inf_dist_forward_nograd_cached(x, weight, cache.get(weight, groups), y, groups)
+    else:
+        _C.inf_dist_forward_nograd(x, weight, y, groups)
+    return y
+
+
+def inf_dist_with_bounds(x, x_lower, x_upper, weight, groups=1, tag=None, cache=None):
     """(y, y_lower, y_upper): the infinity distance of x and the interval bounds of the box (x_lower, x_upper) against
     the same weights: what a layer computes under certification (reference: core/modules/norm_dist.py:30-34, two
     operator calls).  Without gradients the two run as one library call that shares the pre-pass over the weights;
@@ -299,7 +328,11 @@ def inf_dist_with_bounds(x, x_lower, x_upper, weight, groups=1, tag=None):
         x, x_lower, x_upper, weight = (t.contiguous() for t in tensors)
         y = _new_output(x, weight)
         y_lower, y_upper = torch.empty_like(y), torch.empty_like(y)
-        _C.inf_and_bound_forward_nograd(x, x_lower, x_upper, weight, y, y_lower, y_upper, groups)
+        if cache is not None:
+            _C.inf_and_bound_forward_nograd_cached(x, x_lower, x_upper, weight, cache.get(weight, groups), y, y_lower,
+                                                   y_upper, groups)
+        else:
+            _C.inf_and_bound_forward_nograd(x, x_lower, x_upper, weight, y, y_lower, y_upper, groups)
         return y, y_lower, y_upper
     y = norm_dist(x, weight, INF, groups, tag=tag)
     y_lower, y_upper = bound_inf_dist(x_lower, x_upper, weight, groups, tag=tag)

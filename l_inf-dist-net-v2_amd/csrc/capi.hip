@@ -323,6 +323,41 @@ int ndist_inf_and_bound_forward(const float* input, const float* inputL, const f
                                     (hipStream_t)stream);
 }
 
+long long ndist_weight_cache_bytes(int CO, int CI, int G) {
+    Geom s;
+    if (make_geom(1, CO, CI, G, 1, &s)) return 0;
+    return (long long)(weight_seed_floats(s) * sizeof(float));
+}
+
+int ndist_weight_cache_prepare(const float* weight, int CO, int CI, int G, void* cache, ndist_stream_t stream) {
+    NDIST_REQUIRE(weight); NDIST_REQUIRE(cache);
+    Geom s;
+    if (int rc = make_geom(1, CO, CI, G, 1, &s)) return rc;
+    WeightSeeds ws{};
+    return launch_weight_seeds(weight, s, static_cast<float*>(cache), nullptr, 0, (hipStream_t)stream, &ws);
+}
+
+int ndist_inf_dist_forward_nograd_cached(const float* input, const float* weight, const void* cache, int B, int CO, int CI,
+                                         int G, int HW, float* output, ndist_stream_t stream) {
+    NDIST_REQUIRE(input); NDIST_REQUIRE(weight); NDIST_REQUIRE(cache); NDIST_REQUIRE(output);
+    Geom s;
+    if (int rc = make_geom(B, CO, CI, G, HW, &s)) return rc;
+    const WeightSeeds ws = weight_seeds_at(static_cast<float*>(const_cast<void*>(cache)), s);
+    return launch_inf_forward(input, weight, s, output, nullptr, (hipStream_t)stream, nullptr, &ws);
+}
+
+int ndist_inf_and_bound_forward_nograd_cached(const float* input, const float* inputL, const float* inputU,
+                                              const float* weight, const void* cache, int B, int CO, int CI, int G, int HW,
+                                              float* output, float* outputL, float* outputU, ndist_stream_t stream) {
+    NDIST_REQUIRE(input); NDIST_REQUIRE(inputL); NDIST_REQUIRE(inputU); NDIST_REQUIRE(weight); NDIST_REQUIRE(cache);
+    NDIST_REQUIRE(output); NDIST_REQUIRE(outputL); NDIST_REQUIRE(outputU);
+    Geom s;
+    if (int rc = make_geom(B, CO, CI, G, HW, &s)) return rc;
+    const WeightSeeds ws = weight_seeds_at(static_cast<float*>(const_cast<void*>(cache)), s);
+    return launch_inf_bound_forward(input, inputL, inputU, weight, s, output, nullptr, outputL, outputU, nullptr, nullptr,
+                                    (hipStream_t)stream, &ws);
+}
+
 int ndist_unfold_forward(const float* input, int B, int C, int H, int W, int kernel_h, int kernel_w, int dilation_h,
                          int dilation_w, int padding_h, int padding_w, int stride_h, int stride_w, float* output,
                          ndist_stream_t stream) {

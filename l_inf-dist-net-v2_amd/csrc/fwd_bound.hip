@@ -249,10 +249,12 @@ int launch_bound_forward(const float* xl, const float* xu, const float* w, const
 // weights, reference: core/modules/norm_dist.py:30-34): on problems large enough for the k-tile skipping variants the
 // pre-pass over w (the largest of the pre-passes: it reads all of w) runs once and serves both operators.
 int launch_inf_bound_forward(const float* x, const float* xl, const float* xu, const float* w, const Geom& s, float* out,
-                             int32_t* pos, float* yl, float* yu, int32_t* pl, int32_t* pu, hipStream_t st) {
-    if (!seeded_forward_applies(s) && !(hot_forward_applies(s) && hot_alone_applies(s))) {
-        const int rc = launch_inf_forward(x, w, s, out, pos, st);
-        return rc ? rc : launch_bound_forward(xl, xu, w, s, yl, yu, pl, pu, st);
+                             int32_t* pos, float* yl, float* yu, int32_t* pl, int32_t* pu, hipStream_t st,
+                             const WeightSeeds* cached) {
+    if (cached != nullptr || (!seeded_forward_applies(s) && !(hot_forward_applies(s) && hot_alone_applies(s)))) {
+        // (cached: the caller keeps the pre-pass over w between calls; problems that use none ignore it)
+        const int rc = launch_inf_forward(x, w, s, out, pos, st, nullptr, cached);
+        return rc ? rc : launch_bound_forward(xl, xu, w, s, yl, yu, pl, pu, st, nullptr, cached);
     }
     float* block = nullptr;
     NDIST_HIP_TRY(scratch_alloc((void**)&block, weight_seed_floats(s) * sizeof(float), st));

@@ -385,13 +385,20 @@ size_t weight_seed_floats(const Geom& s) {
     return (2 + (size_t)ceil_div(s.CIg, 32)) * ((size_t)s.COg * s.G);
 }
 
+WeightSeeds weight_seeds_at(float* base, const Geom& s) {
+    const long wrows = (long)s.COg * s.G;
+    WeightSeeds ws{};
+    ws.seed_w = base;
+    ws.seed_wk = reinterpret_cast<int32_t*>(base + wrows);
+    ws.tile_w = reinterpret_cast<float*>(ws.seed_wk + wrows);
+    return ws;
+}
+
 int launch_weight_seeds(const float* w, const Geom& s, float* base, const int* gate, int gate_limit, hipStream_t st,
                         WeightSeeds* out) {
     const long wrows = (long)s.COg * s.G;
     const int ntile = ceil_div(s.CIg, 32);
-    out->seed_w = base;
-    out->seed_wk = reinterpret_cast<int32_t*>(base + wrows);
-    out->tile_w = reinterpret_cast<float*>(out->seed_wk + wrows);
+    *out = weight_seeds_at(base, s);
     const SeedSide sw{w, nullptr, wrows, s.CIg, out->seed_w, out->seed_wk, out->tile_w, nullptr, nullptr};
     hipLaunchKernelGGL(norm_seed_kernel, dim3((unsigned)((wrows + 3) / 4)), dim3(256), 0, st, sw, SeedSide{}, (int)((wrows + 3) / 4),
                        ntile, gate, gate_limit, (int*)nullptr);

@@ -133,6 +133,7 @@ struct WeightSeeds {
 size_t seed_scratch_floats(const Geom& s);
 size_t bound_seed_scratch_floats(const Geom& s);  // with the second seed array and the row statistics of the box
 size_t weight_seed_floats(const Geom& s);
+WeightSeeds weight_seeds_at(float* base, const Geom& s);  // the three arrays inside weight_seed_floats(s) floats
 int launch_weight_seeds(const float* w, const Geom& s, float* base, const int* gate, int gate_limit, hipStream_t st,
                         WeightSeeds* out);
 // `wpre`: weight rows already done by launch_weight_seeds (their part of `base` then stays unused)
@@ -271,7 +272,8 @@ int launch_bound_forward(const float* xl, const float* xu, const float* w, const
 bool seeded_forward_applies(const Geom& s);
 // the distance of x and the interval bounds of (xl, xu) against the same weights, pre-passes over w shared
 int launch_inf_bound_forward(const float* x, const float* xl, const float* xu, const float* w, const Geom& s, float* out,
-                             int32_t* pos, float* yl, float* yu, int32_t* pl, int32_t* pu, hipStream_t st);
+                             int32_t* pos, float* yl, float* yu, int32_t* pl, int32_t* pu, hipStream_t st,
+                             const WeightSeeds* cached = nullptr);
 int launch_norm_forward(const float* x, const float* w, const float* max_in, const Geom& s, float* out, float p,
                         hipStream_t st);
 // on images: s describes the unfolded problem, the kernels extract the patches themselves
