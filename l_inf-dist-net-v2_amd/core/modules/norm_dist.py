@@ -64,31 +64,6 @@ class NormDistBase(nn.Module):
         return x, lower, upper
 
 
-class NormDist(NormDistBase):
-    """Fully-connected distance layer on [B, C] tensors (reference: core/modules/norm_dist.py:42-63).
-    `identity_val` plants -identity_val on the wrapped diagonal when the layer does not shrink."""
-
-    def __init__(self, in_features, out_features, groups=1, bias=True, identity_val=None, **kwargs):
-        super().__init__(in_features, out_features, groups=groups, bias=bias, **kwargs)
-        self.in_features = in_features
-        self.out_features = out_features
-        if identity_val is not None and in_features <= out_features:
-            rows = torch.arange(out_features)
-            with torch.no_grad():
-                self.weight[rows, rows % (in_features // groups)] = -identity_val
-
-    def forward(self, x=None, lower=None, upper=None):
-        triple = apply_if_not_none((x, lower, upper), lambda t: t.unsqueeze(-1))
-        triple = super().forward(*triple)
-        return apply_if_not_none(triple, lambda t: t.squeeze(-1))
-
-    def extra_repr(self):
-        s = 'in_features={}, out_features={}, bias={}'.format(self.in_features, self.out_features, self.bias is not None)
-        if self.groups != 1:
-            s += ', groups={}'.format(self.groups)
-        return s
-
-
 class NormDistConv(NormDistBase):
     """Convolutional distance layer on [B, C, H, W]: patches are unfolded to [B, C*kh*kw, H'*W'] and fed to the
     same operator (reference: core/modules/norm_dist.py:66-110)."""
@@ -99,16 +74,14 @@ class NormDistConv(NormDistBase):
             kernel_size = (kernel_size, kernel_size)
         assert in_channels % groups == 0
         super().__init__(in_channels * kernel_size[0] * kernel_size[1], out_channels, groups=groups, bias=bias, **kwargs)
-        self.in_channels = in_channels
-        self.out_channels = out_channels
-        self.kernel_size = kernel_size
-        self.stride = stride
-        self.padding = padding
-        self.dilation = dilation
+        self.in_channels, self.out_channels = in_channels, out_channels
+        self.kernel_size, self.stride, self.padding, self.dilation = kernel_size, stride, padding, dilation
         if identity_val is not None and in_channels <= out_channels:
-            taps = self.weight.data.view(out_channels, -1, *kernel_size)
-            rows = torch.arange(out_channels)
-            taps[rows, rows % (in_channels // groups), kernel_size[0] // 2, kernel_size[1] // 2] = -identity_val
+            # -identity_val at the centre tap of the wrapped diagonal channel
+            co = torch.arange(out_channels)
+            with torch.no_grad():
+                self.weight.view(out_channels, -1, *kernel_size)[
+                    co, co % (in_channels // groups), kernel_size[0] // 2, kernel_size[1] // 2] = -identity_val
 
     def forward(self, x=None, lower=None, upper=None):
         # the operators take the images: they unfold them when a gradient is wanted and extract the patches inside
@@ -128,13 +101,37 @@ class NormDistConv(NormDistBase):
         return apply_if_not_none((x, lower, upper), lambda t: t.view(t.size(0), -1, h, w))
 
     def extra_repr(self):
-        s = '{in_channels}, {out_channels}, kernel_size={kernel_size}, stride={stride}'
-        if self.padding != 0:
-            s += ', padding={padding}'
-        if self.dilation != 1:
-            s += ', dilation={dilation}'
-        if self.groups != 1:
-            s += ', groups={groups}'
+        text = ['%d, %d' % (self.in_channels, self.out_channels), 'kernel_size=%s' % (self.kernel_size,),
+                'stride=%s' % (self.stride,)]
+        # non-default settings only
+        for name, default in (('padding', 0), ('dilation', 1), ('groups', 1)):
+            if getattr(self, name) != default:
+                text.append('%s=%s' % (name, getattr(self, name)))
         if self.bias is None:
-            s += ', bias=False'
-        return s.format(**self.__dict__)
+            text.append('bias=False')
+        return ', '.join(text)
+
+
+class NormDist(NormDistBase):
+    """Fully-connected distance layer on [B, C] tensors (reference: core/modules/norm_dist.py:42-63).
+    `identity_val` plants -identity_val on the wrapped diagonal when the layer does not shrink."""
+
+    def __init__(self, in_features, out_features, groups=1, bias=True, identity_val=None, **kwargs):
+        super().__init__(in_features, out_features, groups=groups, bias=bias, **kwargs)
+        self.in_features = in_features
+        self.out_features = out_features
+        if identity_val is not None and in_features <= out_features:
+            rows = torch.arange(out_features)
+            with torch.no_grad():
+                self.weight[rows, rows % (in_features // groups)] = -identity_val
+
+    def forward(self, x=None, lower=None, upper=None):
+        triple = apply_if_not_none((x, lower, upper), lambda t: t.unsqueeze(-1))
+        triple = super().forward(*triple)
+        return apply_if_not_none(triple, lambda t: t.squeeze(-1))
+
+    def extra_repr(self):
+        shown = [('in_features', self.in_features), ('out_features', self.out_features), ('bias', self.bias is not None)]
+        if self.groups != 1:
+            shown.append(('groups', self.groups))
+        return ', '.join('%s=%s' % item for item in shown)
