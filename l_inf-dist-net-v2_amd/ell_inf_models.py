@@ -23,6 +23,38 @@ def _box(x, eps, up, down, model):
     return x, None, None
 
 
+class hinge:
+    """Hinge loss on the worst-case margins: (1 - mix) * mean_b max_c relu(m) + mix * mean relu(m)
+    (reference: main.py:304-310)."""
+
+    def __init__(self, mix=0.25):
+        self.mix = mix
+
+    def __call__(self, outputs, worst_outputs, targets):
+        return hinge_loss(worst_outputs, self.mix)
+
+
+class HybridModel(nn.Module):
+    """Distance layers followed by a small interval-aware MLP head (reference: ell_inf_models.py:49-76)."""
+
+    def __init__(self, depth, width, input_dim, hidden=512, num_classes=10, std=1.0, identity_val=None):
+        super().__init__()
+        kw = {'std': std, 'identity_val': identity_val}
+        pixels = input_dim[0] * input_dim[1] * input_dim[2]
+        sizes = [pixels] + [width] * (depth - 2)
+        self.fc_dist = BoundSequential(*[NormDist(a, b, bias=False, mean_shift=True, **kw)
+                                         for a, b in zip(sizes[:-1], sizes[1:])])
+        self.fc_linear = BoundSequential(BoundLinear(width, hidden, bias=True), BoundTanh())
+        self.fc_final = BoundFinalLinear(hidden, num_classes, bias=True)
+
+    def forward(self, x=None, targets=None, eps=0, up=None, down=None):
+        paras = apply_if_not_none(_box(x, eps, up, down, self), lambda t: t.view(t.size(0), -1))
+        paras = self.fc_dist(paras)
+        if targets is not None and (paras[1] is None or paras[2] is None):
+            paras = paras[0], paras[0] - eps, paras[0] + eps
+        return self.fc_final(*self.fc_linear(paras), targets=targets)
+
+
 class MLPModel(nn.Module):
     """depth distance layers: pixels -> width -> ... -> width -> num_classes (reference: ell_inf_models.py:16-46).
     Returns -distance as logits; with `targets`, also the worst-case margins of a radius-`eps` ball."""
@@ -48,35 +80,3 @@ class MLPModel(nn.Module):
             lower = x - eps if lower is None else lower
             upper = x + eps if upper is None else upper
         return -x * self.scalar, worst_margin(x, lower, upper, targets, eps)
-
-
-class HybridModel(nn.Module):
-    """Distance layers followed by a small interval-aware MLP head (reference: ell_inf_models.py:49-76)."""
-
-    def __init__(self, depth, width, input_dim, hidden=512, num_classes=10, std=1.0, identity_val=None):
-        super().__init__()
-        kw = {'std': std, 'identity_val': identity_val}
-        pixels = input_dim[0] * input_dim[1] * input_dim[2]
-        sizes = [pixels] + [width] * (depth - 2)
-        self.fc_dist = BoundSequential(*[NormDist(a, b, bias=False, mean_shift=True, **kw)
-                                         for a, b in zip(sizes[:-1], sizes[1:])])
-        self.fc_linear = BoundSequential(BoundLinear(width, hidden, bias=True), BoundTanh())
-        self.fc_final = BoundFinalLinear(hidden, num_classes, bias=True)
-
-    def forward(self, x=None, targets=None, eps=0, up=None, down=None):
-        paras = apply_if_not_none(_box(x, eps, up, down, self), lambda t: t.view(t.size(0), -1))
-        paras = self.fc_dist(paras)
-        if targets is not None and (paras[1] is None or paras[2] is None):
-            paras = paras[0], paras[0] - eps, paras[0] + eps
-        return self.fc_final(*self.fc_linear(paras), targets=targets)
-
-
-class hinge:
-    """Hinge loss on the worst-case margins: (1 - mix) * mean_b max_c relu(m) + mix * mean relu(m)
-    (reference: main.py:304-310)."""
-
-    def __init__(self, mix=0.25):
-        self.mix = mix
-
-    def __call__(self, outputs, worst_outputs, targets):
-        return hinge_loss(worst_outputs, self.mix)
