@@ -212,7 +212,7 @@ int ndist_inf_and_bound_forward_nograd_cached(const float* input, const float* i
 /* ---- mean shift and bias of a distance layer ------------------------------------------------------------------
  * The reference has no kernel of its own here: every layer follows the operator with MeanShift and a bias add
  * written in torch primitives (core/modules/norm_dist.py:35-38, core/modules/basic_modules.py:121-132).  These two
- * entry points do the same in two or three launches.  Tensors are [B, C, HW] like the operator's outputs.
+ * entry points do the same in one launch (fully connected layout, C % 4 == 0) or two to three.  Tensors are [B, C, HW] like the operator's outputs.
  *   forward:  mean[c] = training ? mean over (b, hw) of x : running_mean[c]   (0 when running_mean is NULL in evaluation)
  *             y* = t* - mean[c] + bias1[c] + bias2[c]     for t* in {x, lower, upper} that are not NULL
  *             training also writes mean_out[c] = mean[c] and running_mean[c] = (1 - momentum) running_mean[c] + momentum mean[c]
