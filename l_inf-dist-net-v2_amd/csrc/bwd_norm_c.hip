@@ -58,6 +58,22 @@ __global__ __launch_bounds__(256) void bwd_gx_fixup_kernel(const float* __restri
     const int rc = (int)(sr % P.nrc);
     const int gs = (int)(sr / P.nrc);
     const int grp = gs / P.nslab, ci0 = (gs - grp * P.nslab) * kBwdSlab;
+    if (s.HW == 1 && s.CIg % 4 == 0 && (reinterpret_cast<uintptr_t>(GX) & 15) == 0) {
+        // four consecutive ci per thread: 16-byte loads of every share, all of them on their way before the first add
+        const int e = e0 + 4 * threadIdx.x;
+        if (e >= rows_per_wg * kBwdSlab) return;
+        const int r = e / kBwdSlab, l = e - r * kBwdSlab;
+        const int m = rc * rows_per_wg + r, ci = ci0 + l;
+        if (m >= s.M || ci >= s.CIg) return;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (long g = g_lo; g <= g_hi; g++) {
+            const int slot = sr == begin(g) / P.ncc ? 0 : 1;
+            const float4 t = *reinterpret_cast<const float4*>(part + ((g * 2 + slot) * rows_per_wg + r) * kBwdSlab + l);
+            v = make_float4(v.x + t.x, v.y + t.y, v.z + t.z, v.w + t.w);
+        }
+        *reinterpret_cast<float4*>(GX + x_off(s, m, grp, ci, 0)) = v;
+        return;
+    }
     for (int e = e0 + threadIdx.x; e < min(e0 + 1024, rows_per_wg * kBwdSlab); e += 256) {
         const int r = e / kBwdSlab, l = e - r * kBwdSlab;
         const int m = rc * rows_per_wg + r, ci = ci0 + l;
