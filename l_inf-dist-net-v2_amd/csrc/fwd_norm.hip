@@ -606,7 +606,7 @@ static int launch_row_scaled(FwdParams P, float* scratch, hipStream_t st) {
     hipLaunchKernelGGL(row_scale_kernel, dim3((unsigned)((rows_x + 255) / 256)), dim3(256), 0, st, rx, rows_x, rw, rows_w, P.p, c);
     if (hip_failed(hipGetLastError())) return 4;
     P.aux = c;
-    const int rc = launch_fwd<OpRowScaled, CfgWide4, CfgBig, CfgSmall, CfgWide>(P, st);
+    const int rc = launch_fwd<OpRowScaled, CfgWide4, CfgBig, CfgSmall, CfgWide, CfgLow32, CfgLow16>(P, st);
     if (rc) return rc;
     const long total = rows_x * s.COg;
     const unsigned grid = (unsigned)std::min<long>((total + 255) / 256, 4096);
@@ -616,7 +616,7 @@ static int launch_row_scaled(FwdParams P, float* scratch, hipStream_t st) {
 
 template <int IP>
 static int launch_sum(const FwdParams& P, hipStream_t st) {
-    return launch_fwd<OpSum<IP>, CfgWide4, CfgBig, CfgSmall, CfgWide>(P, st);
+    return launch_fwd<OpSum<IP>, CfgWide4, CfgBig, CfgSmall, CfgWide, CfgLow32, CfgLow16>(P, st);
 }
 
 int launch_norm_forward(const float* x, const float* w, const float* max_in, const Geom& s, float* out, float p,
@@ -642,7 +642,7 @@ int launch_norm_forward(const float* x, const float* w, const float* max_in, con
             float* rs = nullptr;
             if (!scaled || scratch_alloc((void**)&rs, row_scaled_scratch_floats(s) * sizeof(float), st) != hipSuccess) {
                 (void)hipGetLastError();
-                return launch_fwd<OpNormalized<false>, CfgWideT, CfgMid, CfgSmall>(P, st);
+                return launch_fwd<OpNormalized<false>, CfgWideT, CfgMid, CfgSmall, CfgLow32, CfgLow16>(P, st);
             }
             int rc = launch_row_scaled(P, rs, st);
             if (hip_failed(scratch_free(rs, st)) && !rc) rc = 4;
@@ -654,7 +654,7 @@ int launch_norm_forward(const float* x, const float* w, const float* max_in, con
         const size_t nskip = kProbeScratchFloats + seed_scratch_floats(s);
         if (scratch_alloc((void**)&scratch, (nskip + (scaled ? row_scaled_scratch_floats(s) : 0)) * sizeof(float), st) != hipSuccess) {
             (void)hipGetLastError();  // no scratch (out of memory, or a stream under capture): the plain kernel needs none
-            return launch_fwd<OpNormalized<false>, CfgWideT, CfgMid, CfgSmall>(P, st);
+            return launch_fwd<OpNormalized<false>, CfgWideT, CfgMid, CfgSmall, CfgLow32, CfgLow16>(P, st);
         }
         int* gate = reinterpret_cast<int*>(scratch);
         int rc = launch_norm_probe_steps(x, w, s, P.thr, scratch, st);
@@ -677,7 +677,7 @@ int launch_norm_forward(const float* x, const float* w, const float* max_in, con
         if (!rc) {
             P.gate_sense = 0;
             P.aux = nullptr;
-            rc = scaled ? launch_row_scaled(P, scratch + nskip, st) : launch_fwd<OpNormalized<false>, CfgWideT, CfgMid, CfgSmall>(P, st);
+            rc = scaled ? launch_row_scaled(P, scratch + nskip, st) : launch_fwd<OpNormalized<false>, CfgWideT, CfgMid, CfgSmall, CfgLow32, CfgLow16>(P, st);
         }
         if (hip_failed(scratch_free(scratch, st)) && !rc) rc = 4;
         return rc;
