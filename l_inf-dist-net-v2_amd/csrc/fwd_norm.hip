@@ -606,7 +606,7 @@ static int launch_row_scaled(FwdParams P, float* scratch, hipStream_t st) {
     hipLaunchKernelGGL(row_scale_kernel, dim3((unsigned)((rows_x + 255) / 256)), dim3(256), 0, st, rx, rows_x, rw, rows_w, P.p, c);
     if (hip_failed(hipGetLastError())) return 4;
     P.aux = c;
-    const int rc = launch_fwd<OpRowScaled, CfgWide4, CfgBig, CfgSmall, CfgWide, CfgLow32, CfgLow16>(P, st);
+    const int rc = launch_fwd<OpRowScaled, CfgWide4, CfgBig, CfgSmall, CfgWide, CfgLow32, CfgLow16, CfgWide4H>(P, st);
     if (rc) return rc;
     const long total = rows_x * s.COg;
     const unsigned grid = (unsigned)std::min<long>((total + 255) / 256, 4096);
@@ -616,7 +616,7 @@ static int launch_row_scaled(FwdParams P, float* scratch, hipStream_t st) {
 
 template <int IP>
 static int launch_sum(const FwdParams& P, hipStream_t st) {
-    return launch_fwd<OpSum<IP>, CfgWide4, CfgBig, CfgSmall, CfgWide, CfgLow32, CfgLow16>(P, st);
+    return launch_fwd<OpSum<IP>, CfgWide4, CfgBig, CfgSmall, CfgWide, CfgLow32, CfgLow16, CfgWide4H>(P, st);
 }
 
 int launch_norm_forward(const float* x, const float* w, const float* max_in, const Geom& s, float* out, float p,

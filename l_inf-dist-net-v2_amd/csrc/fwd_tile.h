@@ -586,6 +586,9 @@ using CfgSmall = TileCfg<4, 4, 2, 2, 1>;  // 64 x 64, 256 threads
 // 5120 x 5120: 0.166 -> 0.108 ms at 32 rows, 0.162 -> 0.068 ms at 8 and 16)
 using CfgLow32 = TileCfg<4, 4, 1, 4, 1>;  // 32 x 128, 256 threads
 using CfgLow16 = TileCfg<2, 8, 1, 4, 1>;  // 16 x 256, 256 threads
+// 33 to 64 rows: the 1024-thread tile at half height (64 x 80): four waves per SIMD from one workgroup per compute
+// unit, where the 256-thread 64 x 64 tiles leave the SIMDs with two (p = 8 at 64 x 5120 x 5120: 0.176 -> 0.160 ms)
+using CfgWide4H = TileCfg<4, 5, 2, 2, 4, 16>;
 
 // Second step of a split k range: merges the partial accumulators of one output in split order, finalises, stores.
 template <class Op>
@@ -699,7 +702,9 @@ double tile_cost(const Geom& s, int cus, double part_cost) {
     const double alone = Cfg::NT <= 256 && tiles <= cus ? 1.6 : 1.0;
     const double split = Cfg::NT > 256 && ks > 1 ? 1.01 + part_cost * ks : 1.0;  // as in tile_ksplit
     const double few_waves = Cfg::NT <= 256 ? 1.1 : 1.0;
-    return (double)per_cu * Cfg::BM * Cfg::BN * lds * alone * few_waves * split / ks;
+    // measured: at equal padded area the half-height 1024-thread tile is 9 % slower than the full one
+    const double half = std::is_same<Cfg, CfgWide4H>::value ? 1.08 : 1.0;
+    return (double)per_cu * Cfg::BM * Cfg::BN * lds * alone * few_waves * half * split / ks;
 }
 
 }  // namespace ndist
