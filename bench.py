@@ -240,6 +240,7 @@ def run_part(torch, _C, args, xd, wd, gd):
     out8 = out.clone()
     _C.norm_dist_forward(xd, wd, out, 1, 13.7)
     out137 = out.clone()
+    rmean, bmean, shifted = torch.zeros(CO, device=xd.device), torch.empty(CO, device=xd.device), torch.empty_like(out)
     _C.inf_dist_forward(xd, wd, out, pos, 1)
     calls = {
         "p8_fwd": lambda: _C.norm_dist_forward(xd, wd, out, 1, 8.0),
@@ -249,6 +250,8 @@ def run_part(torch, _C, args, xd, wd, gd):
         "inf_fwd": lambda: _C.inf_dist_forward(xd, wd, out, pos, 1),
         "inf_fwd_nograd": lambda: _C.inf_dist_forward_nograd(xd, wd, out, 1),
         "inf_bwd": lambda: _C.inf_dist_backward_input_weight(gd, pos, gx, gw, 1),
+        # what follows the operator in a layer: batch mean, moving average, subtraction (one launch)
+        "mean_shift": lambda: _C.mean_shift_forward(out8, None, None, True, 0.1, rmean, None, None, bmean, shifted, None, None),
     }
     if args.part == "copy":
         # calibration for the FETCH_SIZE / WRITE_SIZE counters: a plain device copy of 256 MiB (read once, written once)
@@ -276,7 +279,7 @@ def main():
     ap.add_argument("--cpu-cols", type=int, default=1024, help="output features of the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-other", action="store_true", help="skip the secondary workloads (general p, IBP, MLP, conv)")
     ap.add_argument("--part", default="all",
-                    choices=["all", "p8_fwd", "p8_bwd", "p13.7_fwd", "p13.7_bwd", "inf_fwd", "inf_fwd_nograd", "inf_bwd", "copy", "other"],
+                    choices=["all", "p8_fwd", "p8_bwd", "p13.7_fwd", "p13.7_bwd", "mean_shift", "inf_fwd", "inf_fwd_nograd", "inf_bwd", "copy", "other"],
                     help="profiling aid: run only one entry point of the step, --steps times, on pre-allocated outputs")
     ap.add_argument("--batch", type=int, default=B, help="with --part: rows of the batch to use (e.g. 64)")
     args = ap.parse_args()
