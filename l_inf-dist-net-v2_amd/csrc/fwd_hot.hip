@@ -183,6 +183,20 @@ __global__ __launch_bounds__(1024) void hot_plan_kernel(const float* __restrict_
     }
 }
 
+// Value of the partner lane in a merge of the eight lanes that share a row: step 1 and 2 are the butterfly inside a
+// quad (quad_perm), step 4 pairs lane i of one quad with lane 7 - i of the other (row_half_mirror) -- by then all four
+// lanes of a quad hold the same state, so any lane of the other quad will do.  DPP moves: no LDS round trip.
+template <typename T>
+__device__ __forceinline__ T partner8(T v, int d) {
+    static_assert(sizeof(T) == 4, "32-bit values");
+    const int i = __builtin_bit_cast(int, v);
+    int r;
+    if (d == 1) r = __builtin_amdgcn_update_dpp(0, i, 0xB1, 0xf, 0xf, true);        // quad_perm [1, 0, 3, 2]
+    else if (d == 2) r = __builtin_amdgcn_update_dpp(0, i, 0x4E, 0xf, 0xf, true);   // quad_perm [2, 3, 0, 1]
+    else r = __builtin_amdgcn_update_dpp(0, i, 0x141, 0xf, 0xf, true);              // row_half_mirror
+    return __builtin_bit_cast(T, r);
+}
+
 // The two operators as policies of the walk: per-output state, one pair, the merge of two lanes' states (the larger
 // value, among equal values the lower k; "nothing found" carries the operator's initial code, which no found pair
 // can tie with because a pair must beat the floor strictly), the outputs.
@@ -200,9 +214,9 @@ struct HotInf {  // out = max(1e-10, max_k |x - w|), code = k | sign flag (core/
         }
     }
     __device__ static __forceinline__ void merge_xor(State& a, int d) {
-        const float ob = __shfl_xor(a.best, d, 64);
+        const float ob = partner8(a.best, d);
         if constexpr (TRACK) {
-            const uint32_t oc = __shfl_xor(a.code, d, 64);
+            const uint32_t oc = partner8(a.code, d);
             const bool take = ob > a.best || (ob == a.best && (oc & ~kSignBit) < (a.code & ~kSignBit));
             a.best = take ? ob : a.best;
             a.code = take ? oc : a.code;
@@ -239,9 +253,9 @@ struct HotBound {  // interval bounds (core/cuda/bound_inf_dist_cuda.cu:63,148-1
         }
     }
     __device__ static __forceinline__ void merge_xor(State& a, int d) {
-        const float ol = __shfl_xor(a.lo, d, 64), oh = __shfl_xor(a.hi, d, 64);
+        const float ol = partner8(a.lo, d), oh = partner8(a.hi, d);
         if constexpr (TRACK) {
-            const uint32_t cl = __shfl_xor(a.wl, d, 64), cu = __shfl_xor(a.wu, d, 64);
+            const uint32_t cl = partner8(a.wl, d), cu = partner8(a.wu, d);
             const bool tl = ol < a.lo || (ol == a.lo && (cl & ~kSignBit) < (a.wl & ~kSignBit));
             const bool tu = oh > a.hi || (oh == a.hi && (cu & ~kSignBit) < (a.wu & ~kSignBit));
             a.lo = tl ? ol : a.lo;
