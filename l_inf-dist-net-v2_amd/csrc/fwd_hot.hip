@@ -94,7 +94,6 @@ __global__ __launch_bounds__(1024) void hot_plan_kernel(const float* __restrict_
     __shared__ int is_last;
     __shared__ long long tot[2];
     if (threadIdx.x < 2) { cnt[threadIdx.x] = 0; tot[threadIdx.x] = 0; }
-    hot_group_maxima(seed_x, seed_w, s, sm);
     const long rows = (long)s.M * s.G, wrows = (long)s.COg * s.G;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     constexpr int R = kPlanRowsPerWave;
@@ -105,42 +104,67 @@ __global__ __launch_bounds__(1024) void hot_plan_kernel(const float* __restrict_
     long rr[R];
     int count[R];
     uint32_t nonzero[R];  // bit i: mask word i of the row has a hot tile (first word of the row's record)
+    float own[R], fh[R], fl[R];
 #pragma unroll
     for (int i = 0; i < R; i++) {
         const long r = (long)blockIdx.x * kPlanRows + wave * R + i;
         valid[i] = r < rows + wrows;  // wave-uniform
         isw[i] = r >= rows;
         rr[i] = !valid[i] ? 0 : (isw[i] ? r - rows : r);
-        const int g = isw[i] ? (int)(rr[i] / s.COg) : (int)(rr[i] % s.G);
-        const float own = fabsf(isw[i] ? seed_w[valid[i] ? rr[i] : 0] : seed_x[rr[i]]);
-        const float other = __uint_as_float(sm[isw[i] ? g : s.G + g]);
-        thr[i] = hot_threshold(own, other);
-        if (!isw[i] && far_hi != nullptr) {
-            // interval bounds, rows of the box: the two reductions have their own lower bounds, far_hi - RW for the
-            // upper one and far_lo - RW for the lower one; a tile is dead when it is dead for both
-            const double tu = hot_threshold(far_hi[rr[i]], other), tl = hot_threshold(far_lo[rr[i]], other);
-            thr[i] = own == own ? (tu < tl ? tu : tl) : -__builtin_inf();
-        }
         tm[i] = (isw[i] ? tile_w : tile_x) + rr[i] * ntile;
         mk[i] = (isw[i] ? mask_w : mask_x) + rr[i] * (nword + 1);
         count[i] = 0;
         nonzero[i] = 0u;
+        own[i] = fabsf(isw[i] ? seed_w[rr[i]] : seed_x[rr[i]]);
+        fh[i] = fl[i] = 0.f;
+        if (!isw[i] && far_hi != nullptr) {
+            fh[i] = far_hi[rr[i]];
+            fl[i] = far_lo[rr[i]];
+        }
     }
-    for (int t0 = 0; t0 < nword * 32; t0 += 64) {
-        const int t = t0 + lane;
-        float v[R];
+    // The tile maxima of four steps (256 tiles of each row) are requested together, and the first such batch before
+    // the group maxima are formed: the kernel is a chain of memory latencies, this leaves one for everything up to 8192 k.
+    constexpr int STEPS = 4;
+    float v[STEPS][R];
+    auto fetch = [&](int t00) {
 #pragma unroll
-        for (int i = 0; i < R; i++) v[i] = valid[i] && t < ntile ? tm[i][t] : 0.f;
+        for (int q = 0; q < STEPS; q++) {
+            const int t = t00 + 64 * q + lane;
 #pragma unroll
-        for (int i = 0; i < R; i++) {
-            const bool hot = valid[i] && t < ntile && !((double)v[i] < thr[i]);
-            const unsigned long long bits = __builtin_amdgcn_ballot_w64(hot);
-            count[i] += __popcll(bits);
-            const int wi = t0 >> 5;
-            nonzero[i] |= ((uint32_t)bits != 0u ? 1u << (wi & 31) : 0u) | ((bits >> 32) != 0ull ? 1u << ((wi + 1) & 31) : 0u);
-            if (lane == 0 && valid[i]) {
-                mk[i][1 + wi] = (uint32_t)bits;
-                if (wi + 1 < nword) mk[i][2 + wi] = (uint32_t)(bits >> 32);
+            for (int i = 0; i < R; i++) v[q][i] = valid[i] && t < ntile ? tm[i][t] : 0.f;
+        }
+    };
+    fetch(0);
+    hot_group_maxima(seed_x, seed_w, s, sm);
+#pragma unroll
+    for (int i = 0; i < R; i++) {
+        const int g = isw[i] ? (int)(rr[i] / s.COg) : (int)(rr[i] % s.G);
+        const float other = __uint_as_float(sm[isw[i] ? g : s.G + g]);
+        thr[i] = hot_threshold(own[i], other);
+        if (!isw[i] && far_hi != nullptr) {
+            // interval bounds, rows of the box: the two reductions have their own lower bounds, far_hi - RW for the
+            // upper one and far_lo - RW for the lower one; a tile is dead when it is dead for both
+            const double tu = hot_threshold(fh[i], other), tl = hot_threshold(fl[i], other);
+            thr[i] = own[i] == own[i] ? (tu < tl ? tu : tl) : -__builtin_inf();
+        }
+    }
+    for (int t00 = 0; t00 < nword * 32; t00 += 64 * STEPS) {
+        if (t00 > 0) fetch(t00);
+#pragma unroll
+        for (int q = 0; q < STEPS; q++) {
+            const int t0 = t00 + 64 * q, t = t0 + lane;
+            if (t0 >= nword * 32) break;  // the same for all lanes
+#pragma unroll
+            for (int i = 0; i < R; i++) {
+                const bool hot = valid[i] && t < ntile && !((double)v[q][i] < thr[i]);
+                const unsigned long long bits = __builtin_amdgcn_ballot_w64(hot);
+                count[i] += __popcll(bits);
+                const int wi = t0 >> 5;
+                nonzero[i] |= ((uint32_t)bits != 0u ? 1u << (wi & 31) : 0u) | ((bits >> 32) != 0ull ? 1u << ((wi + 1) & 31) : 0u);
+                if (lane == 0 && valid[i]) {
+                    mk[i][1 + wi] = (uint32_t)bits;
+                    if (wi + 1 < nword) mk[i][2 + wi] = (uint32_t)(bits >> 32);
+                }
             }
         }
     }
@@ -160,17 +184,22 @@ __global__ __launch_bounds__(1024) void hot_plan_kernel(const float* __restrict_
         is_last = atomicAdd(&dec[3], 1) == (int)gridDim.x - 1;
     }
     __syncthreads();
-    if (!is_last) return;
+    if (!is_last || wave != 0) return;
+    // the last workgroup's first wave adds the counts up (butterfly over the lanes) and decides
     __threadfence();
     long long cx = 0, cw = 0;
-    for (int b = threadIdx.x; b < (int)gridDim.x; b += blockDim.x) {
+    for (int b = lane; b < (int)gridDim.x; b += 64) {
         cx += __atomic_load_n(&partial[2 * b], __ATOMIC_RELAXED);
         cw += __atomic_load_n(&partial[2 * b + 1], __ATOMIC_RELAXED);
     }
-    if (cx != 0) atomicAdd((unsigned long long*)&tot[0], (unsigned long long)cx);
-    if (cw != 0) atomicAdd((unsigned long long*)&tot[1], (unsigned long long)cw);
-    __syncthreads();
-    if (threadIdx.x == 0) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        cx += __shfl_xor(cx, d, 64);
+        cw += __shfl_xor(cw, d, 64);
+    }
+    if (lane == 0) {
+        tot[0] = cx;
+        tot[1] = cw;
         const long long costx = tot[0] * s.COg, costw = tot[1] * s.M;
         const long long total = (long long)s.M * s.G * s.COg * ntile;
         int choice = costx <= costw ? 1 : 2;
