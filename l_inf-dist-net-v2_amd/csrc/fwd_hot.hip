@@ -229,6 +229,17 @@ __device__ __forceinline__ T partner8(T v, int d) {
 // The two operators as policies of the walk: per-output state, one pair, the merge of two lanes' states (the larger
 // value, among equal values the lower k; "nothing found" carries the operator's initial code, which no found pair
 // can tie with because a pair must beat the floor strictly), the outputs.
+// For the merges a code travels as a rank: higher for lower k, sign flag in the lowest bit.  (value, rank) pairs of
+// positive values then order as 64-bit integers -- larger value first, among equal values the lower k -- and a merge
+// step is one 64-bit compare and two selects per reduction.
+__device__ __forceinline__ uint32_t code_to_rank(uint32_t code) { return ((0x7fffffffu - (code & ~kSignBit)) << 1) | (code >> 31); }
+__device__ __forceinline__ uint32_t rank_to_code(uint32_t rank) { return (0x7fffffffu - (rank >> 1)) | (rank << 31); }
+__device__ __forceinline__ bool pair_beats(float ov, uint32_t orank, float v, uint32_t rank) {
+    const unsigned long long a = ((unsigned long long)__float_as_uint(ov) << 32) | orank;
+    const unsigned long long b = ((unsigned long long)__float_as_uint(v) << 32) | rank;
+    return a > b;
+}
+
 template <bool TRACK>
 struct HotInf {  // out = max(1e-10, max_k |x - w|), code = k | sign flag (core/cuda/inf_dist_cuda.cu:131-132,173-177)
     static constexpr int NX = 1, NF = 1, NI = TRACK ? 1 : 0;
@@ -242,11 +253,18 @@ struct HotInf {  // out = max(1e-10, max_k |x - w|), code = k | sign flag (core/
             a.best = fmaxf(a.best, v);
         }
     }
+    // around the merge steps of a state: its code as a rank and back
+    __device__ static __forceinline__ void pre_merge(State& a) {
+        if constexpr (TRACK) a.code = code_to_rank(a.code);
+    }
+    __device__ static __forceinline__ void post_merge(State& a) {
+        if constexpr (TRACK) a.code = rank_to_code(a.code);
+    }
     __device__ static __forceinline__ void merge_xor(State& a, int d) {
         const float ob = partner8(a.best, d);
         if constexpr (TRACK) {
             const uint32_t oc = partner8(a.code, d);
-            const bool take = ob > a.best || (ob == a.best && (oc & ~kSignBit) < (a.code & ~kSignBit));
+            const bool take = pair_beats(ob, oc, a.best, a.code);
             a.best = take ? ob : a.best;
             a.code = take ? oc : a.code;
         } else {
@@ -281,12 +299,28 @@ struct HotBound {  // interval bounds (core/cuda/bound_inf_dist_cuda.cu:63,148-1
             a.hi = fmaxf(a.hi, mx);
         }
     }
+    // around the merge steps of a state: the lower reduction negated (a maximum of positive values like the upper
+    // one), the codes as ranks
+    __device__ static __forceinline__ void pre_merge(State& a) {
+        if constexpr (TRACK) {
+            a.lo = -a.lo;
+            a.wl = code_to_rank(a.wl);
+            a.wu = code_to_rank(a.wu);
+        }
+    }
+    __device__ static __forceinline__ void post_merge(State& a) {
+        if constexpr (TRACK) {
+            a.lo = -a.lo;
+            a.wl = rank_to_code(a.wl);
+            a.wu = rank_to_code(a.wu);
+        }
+    }
     __device__ static __forceinline__ void merge_xor(State& a, int d) {
         const float ol = partner8(a.lo, d), oh = partner8(a.hi, d);
         if constexpr (TRACK) {
             const uint32_t cl = partner8(a.wl, d), cu = partner8(a.wu, d);
-            const bool tl = ol < a.lo || (ol == a.lo && (cl & ~kSignBit) < (a.wl & ~kSignBit));
-            const bool tu = oh > a.hi || (oh == a.hi && (cu & ~kSignBit) < (a.wu & ~kSignBit));
+            const bool tl = pair_beats(ol, cl, a.lo, a.wl);
+            const bool tu = pair_beats(oh, cu, a.hi, a.wu);
             a.lo = tl ? ol : a.lo;
             a.wl = tl ? cl : a.wl;
             a.hi = tu ? oh : a.hi;
@@ -320,7 +354,8 @@ constexpr int kHotRows = 8 * kHotSlots;    // rows of the other side per wave
 template <class P, bool X_OWNS>
 __device__ __forceinline__ void hot_walk(const float* __restrict__ own, const float* __restrict__ oth, long x2off,
                                          long stride, int nrow, const uint32_t* __restrict__ mk, int nword, int K,
-                                         bool vec, typename P::State& res) {
+                                         bool vec, typename P::State& res, bool ahead = false, uint32_t summary = 0,
+                                         uint32_t first_word = 0) {
     using State = typename P::State;
     constexpr bool TWO = P::NX == 2;
     const int lane = threadIdx.x & 63, sub = lane & 7, q = lane >> 3;
@@ -334,8 +369,10 @@ __device__ __forceinline__ void hot_walk(const float* __restrict__ own, const fl
     }
     // mk[0] names the mask words that hold a hot tile (when there are at most 32 of them): usually a single one, so
     // the walk costs two dependent loads instead of one per word
-    uint32_t pending = mk[0];
+    // (`ahead`: the caller has fetched the summary and the first word it names already, for several rows at once)
+    uint32_t pending = ahead ? summary : mk[0];
     int wi = -1;
+    bool first = ahead;
     while (true) {
         if (nword <= 32) {
             if (pending == 0) break;
@@ -344,7 +381,8 @@ __device__ __forceinline__ void hot_walk(const float* __restrict__ own, const fl
         } else if (++wi >= nword) {
             break;
         }
-        uint32_t bits = mk[1 + wi];
+        uint32_t bits = first ? first_word : mk[1 + wi];
+        first = false;
         while (bits != 0) {
             const int k0 = (wi * 32 + __builtin_ctz(bits)) * 32 + 4 * sub;
             bits &= bits - 1;
@@ -389,8 +427,10 @@ __device__ __forceinline__ void hot_walk(const float* __restrict__ own, const fl
     // the eight lanes of a row merge
 #pragma unroll
     for (int j = 0; j < kHotSlots; j++) {
+        P::pre_merge(st[j]);
 #pragma unroll
         for (int d = 1; d < 8; d <<= 1) P::merge_xor(st[j], d);
+        P::post_merge(st[j]);
     }
     res = st[0];
 #pragma unroll
@@ -449,13 +489,31 @@ __global__ __launch_bounds__(256) void hot_kernel(const float* __restrict__ x, l
         const int nb = (int)(id % (unsigned)nnb), g = (int)(id / (unsigned)nnb);
         const int m0 = mb * kHotRows;
         // HW == 1: row m of group g of x starts at (m * G + g) * CIg, consecutive rows are G * CIg apart
+        // The four rows of a wave are walked one after the other, each a chain of dependent loads (summary, mask
+        // word, tile pieces): the summaries of all four, then the first words they name, are fetched up front.
+        const bool ahead = nword <= 32;
+        uint32_t summary[4] = {0u, 0u, 0u, 0u}, word0[4] = {0u, 0u, 0u, 0u};
+        if (ahead) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int n = min(nb * 16 + wave * 4 + i, s.COg - 1);
+                summary[i] = mask_w[((long)g * s.COg + n) * (nword + 1)];
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int n = min(nb * 16 + wave * 4 + i, s.COg - 1);
+                const int w0 = summary[i] != 0u ? __builtin_ctz(summary[i]) : 0;
+                word0[i] = mask_w[((long)g * s.COg + n) * (nword + 1) + 1 + w0];
+            }
+        }
         for (int i = 0; i < 4; i++) {
             const int c = wave * 4 + i, n = nb * 16 + c;
             P::init(res);
             if (n < s.COg) {  // wave-uniform
                 const long wrow = (long)g * s.COg + n;
                 hot_walk<P, false>(w + wrow * s.CIg, x + ((long)m0 * s.G + g) * s.CIg, x2off, (long)s.CIg * s.G,
-                                   min(kHotRows, s.M - m0), mask_w + wrow * (nword + 1), nword, s.CIg, vec != 0, res);
+                                   min(kHotRows, s.M - m0), mask_w + wrow * (nword + 1), nword, s.CIg, vec != 0, res,
+                                   ahead, summary[i], word0[i]);
             }
             P::outputs(res, fv, iv);
             if (reports) {
