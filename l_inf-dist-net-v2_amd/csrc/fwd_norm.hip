@@ -149,6 +149,69 @@ struct SeedSide {
     float* out_hi;
     float* out_lo;
 };
+template <int CTRL>
+__device__ __forceinline__ float lane_swap(float v) {  // data-parallel-primitive move: no LDS traffic
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+// The row's elements through 16-byte loads (1 KiB per wave and instruction), ten loads in flight per lane: a wave
+// alone keeps 10 KiB on its way.  The loads are unconditional (addresses behind the row's end fall back on its last
+// four k): a load under a per-lane condition is split into four 4-byte ones.  The tile maxima of a pass go through
+// LDS so that they leave in whole lines.  BOX: two arrays (interval bounds), the larger magnitude of the two counts.
+template <bool BOX>
+__device__ __forceinline__ void seed_row_wide(const float* __restrict__ xp, const float* __restrict__ xq, int K, int ntile,
+                                              float* __restrict__ tm, int lane, float& best, float& val, int& bk,
+                                              bool& bad, float& far_hi, float& far_lo) {
+    constexpr int U = BOX ? 5 : 10;
+    __shared__ float stage_all[4][8 * U];
+    float* stage = stage_all[threadIdx.x >> 6];
+    for (int k0 = 0; k0 < K; k0 += 256 * U) {
+        float4 a4[U], b4[BOX ? U : 1];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int k = min(k0 + 256 * u + 4 * lane, K - 4);
+            a4[u] = *reinterpret_cast<const float4*>(xp + k);
+            if constexpr (BOX) b4[u] = *reinterpret_cast<const float4*>(xq + k);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int k = k0 + 256 * u + 4 * lane;
+            if (k0 + 256 * u >= K) break;  // wave-uniform
+            float local = 0.f;  // largest magnitude of my four k: they lie in one tile, 8 lanes share a tile
+            if (k < K) {
+                float v[4] = {a4[u].x, a4[u].y, a4[u].z, a4[u].w};
+                const float sum4 = (v[0] + v[1]) + (v[2] + v[3]);
+                bad |= sum4 != sum4;
+                if constexpr (BOX) {
+                    const float v2[4] = {b4[u].x, b4[u].y, b4[u].z, b4[u].w};
+                    const float sum4b = (v2[0] + v2[1]) + (v2[2] + v2[3]);
+                    bad |= sum4b != sum4b;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        float lo = v[j], up = v2[j];
+                        if (lo > up) lo = up = (lo + up) * 0.5f;
+                        far_hi = fmaxf(far_hi, fmaxf(-lo, up));
+                        far_lo = fmaxf(far_lo, fmaxf(lo, -up));
+                        v[j] = fabsf(v2[j]) > fabsf(v[j]) ? v2[j] : v[j];
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    local = fmaxf(local, fabsf(v[j]));
+                    if (fabsf(v[j]) > best) { best = fabsf(v[j]); val = v[j]; bk = k + j; }
+                }
+            }
+            local = fmaxf(local, lane_swap<0xB1>(local));   // quad_perm [1, 0, 3, 2]
+            local = fmaxf(local, lane_swap<0x4E>(local));   // quad_perm [2, 3, 0, 1]
+            local = fmaxf(local, lane_swap<0x141>(local));  // row_half_mirror
+            if ((lane & 7) == 0) stage[8 * u + (lane >> 3)] = local;
+        }
+        __builtin_amdgcn_wave_barrier();
+        const int t0 = k0 >> 5, nt = min(8 * U, ntile - t0);
+        for (int t = lane; t < nt; t += 64) tm[t0 + t] = stage[t];
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
 __device__ __forceinline__ void norm_seed_row(const SeedSide& sd, long r, int ntile) {
     const int lane = threadIdx.x & 63;
     const int K = sd.K;
@@ -160,36 +223,9 @@ __device__ __forceinline__ void norm_seed_row(const SeedSide& sd, long r, int nt
     int bk = 0;
     bool bad = false;  // a NaN in the row (or +inf next to -inf): the pair at the row's seed may not exist
     float far_hi = -__builtin_inff(), far_lo = -__builtin_inff();
-    if (K % 4 == 0 && (uintptr_t)x % 16 == 0 && xq == nullptr) {  // 16-byte loads: 1 KiB per wave and iteration
-        // four loads in flight per lane: a wave alone keeps 4 KiB of the row on its way
-        for (int k0 = 0; k0 < K; k0 += 1024) {
-            float4 v4[4];
-#pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const int k = k0 + 256 * u + 4 * lane;
-                v4[u] = k < K ? *reinterpret_cast<const float4*>(xp + k) : make_float4(0.f, 0.f, 0.f, 0.f);
-            }
-#pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const int k = k0 + 256 * u + 4 * lane;
-                if (k0 + 256 * u >= K) break;  // wave-uniform
-                float local = 0.f;  // largest magnitude of my four k: they lie in one tile, 8 lanes share a tile
-                if (k < K) {
-                    const float v[4] = {v4[u].x, v4[u].y, v4[u].z, v4[u].w};
-                    const float sum4 = (v[0] + v[1]) + (v[2] + v[3]);
-                    bad |= sum4 != sum4;
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        local = fmaxf(local, fabsf(v[j]));
-                        if (fabsf(v[j]) > best) { best = fabsf(v[j]); val = v[j]; bk = k + j; }
-                    }
-                }
-                local = fmaxf(local, __shfl_xor(local, 1, 64));
-                local = fmaxf(local, __shfl_xor(local, 2, 64));
-                local = fmaxf(local, __shfl_xor(local, 4, 64));
-                if ((lane & 7) == 0 && k < K) tm[k >> 5] = local;
-            }
-        }
+    if (K % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)sd.x2 % 16 == 0) {
+        if (xq == nullptr) seed_row_wide<false>(xp, xq, K, ntile, tm, lane, best, val, bk, bad, far_hi, far_lo);
+        else seed_row_wide<true>(xp, xq, K, ntile, tm, lane, best, val, bk, bad, far_hi, far_lo);
     } else {
         for (int k0 = 0; k0 < K; k0 += 64) {
             const int k = k0 + lane;
