@@ -3,7 +3,9 @@
 // each walk the whole k range alone; here the k range is spread over the 64 lanes of a wave instead: one wave owns
 // 2 rows x 4 co, every lane takes 4 consecutive k of each 256-wide step (one 16-byte load per operand row, 1 KiB
 // contiguous per wave), accumulates with the same operator policies as the tiled kernel, and the lanes are merged
-// with a butterfly of cross-lane shuffles at the end.  No LDS, no barriers.  Fully-connected layout only.
+// with a butterfly of cross-lane shuffles at the end.  The four waves of a workgroup share one such block of outputs
+// and take every fourth step each (a wave alone would walk K / 256 dependent memory latencies: 37 us for the 512 x 10
+// layer); their results meet in LDS after the one barrier of the kernel.  Fully-connected layout only.
 //
 // Arg-max bookkeeping: a lane's "tile" is its 4 consecutive k of one step (tile index step * 64 + lane, so tiles
 // are ordered like their k); the rescan kernels then run with a tile length of 4.
@@ -34,10 +36,8 @@ __global__ __launch_bounds__(256) void fwd_skinny_kernel(const FwdParams P, int 
     using Acc = typename Op::Acc;
     if (gate_closed(P)) return;
     const Geom& s = P.s;
-    const int lane = threadIdx.x & 63;
-    long wid = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const long nw = (long)s.G * nrp * ncq;
-    if (wid >= nw) return;  // whole waves leave; there is no barrier in this kernel
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    long wid = blockIdx.x;  // one block of outputs per workgroup: nobody leaves before the barrier
     const int cq = (int)(wid % ncq);
     wid /= ncq;
     const int rp = (int)(wid % nrp), g = (int)(wid / nrp);
@@ -47,7 +47,7 @@ __global__ __launch_bounds__(256) void fwd_skinny_kernel(const FwdParams P, int 
 #pragma unroll
     for (int r = 0; r < R; r++)
 #pragma unroll
-        for (int j = 0; j < TN; j++) Op::init(acc[r][j], P, lane == 0 ? 0 : 1, m0 + r, n0 + j, g);
+        for (int j = 0; j < TN; j++) Op::init(acc[r][j], P, (lane | wave) == 0 ? 0 : 1, m0 + r, n0 + j, g);
 
     const float* xrow[NX][R];
     const float* wrow[TN];
@@ -105,14 +105,15 @@ __global__ __launch_bounds__(256) void fwd_skinny_kernel(const FwdParams P, int 
         }
     };
 
+    // my steps: wave, wave + 4, ... (the workgroup reads 4 KiB of every operand row at a time)
     const int nsteps = ceil_div(K, 256);
-    fetch(0, lane * 4);
-    for (int it = 0; it < nsteps; it += 2) {
-        if (it + 1 < nsteps) fetch(1, (it + 1) * 256 + lane * 4);
+    if (wave < nsteps) fetch(0, wave * 256 + lane * 4);
+    for (int it = wave; it < nsteps; it += 8) {
+        if (it + 4 < nsteps) fetch(1, (it + 4) * 256 + lane * 4);
         compute(0, it * 64 + lane);
-        if (it + 1 < nsteps) {
-            if (it + 2 < nsteps) fetch(0, (it + 2) * 256 + lane * 4);
-            compute(1, (it + 1) * 64 + lane);
+        if (it + 4 < nsteps) {
+            if (it + 8 < nsteps) fetch(0, (it + 8) * 256 + lane * 4);
+            compute(1, (it + 4) * 64 + lane);
         }
     }
 
@@ -124,6 +125,26 @@ __global__ __launch_bounds__(256) void fwd_skinny_kernel(const FwdParams P, int 
 #pragma unroll
             for (int j = 0; j < TN; j++) {
                 const Acc other = shuffle_xor_acc(acc[r][j], mask);
+                Op::merge(acc[r][j], other, P);
+            }
+
+    // ---- merge the waves
+    __shared__ Acc part[3][R][TN];
+    if (wave != 0 && lane == 0) {
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) part[wave - 1][r][j] = acc[r][j];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int q = 0; q < 3; q++)
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                const Acc other = part[q][r][j];
                 Op::merge(acc[r][j], other, P);
             }
 
@@ -165,7 +186,7 @@ int launch_skinny(FwdParams P, hipStream_t st, int* chosen_kt) {
     const int nrp = ceil_div(s.M, kSkinnyRows), ncq = ceil_div(s.COg, kSkinnyCols);
     const long nw = (long)s.G * nrp * ncq;
     KernelTimer timer(st);
-    hipLaunchKernelGGL((fwd_skinny_kernel<Op>), dim3((unsigned)((nw + 3) / 4)), dim3(256), 0, st, P, nrp, ncq);
+    hipLaunchKernelGGL((fwd_skinny_kernel<Op>), dim3((unsigned)nw), dim3(256), 0, st, P, nrp, ncq);
     return hip_failed(hipGetLastError()) ? 4 : 0;
 }
 
