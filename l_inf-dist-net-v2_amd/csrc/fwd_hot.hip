@@ -241,7 +241,8 @@ __device__ __forceinline__ bool pair_beats(float ov, uint32_t orank, float v, ui
 }
 
 template <bool TRACK>
-struct HotInf {  // out = max(1e-10, max_k |x - w|), code = k | sign flag (core/cuda/inf_dist_cuda.cu:131-132,173-177)
+struct HotInf {
+    static constexpr int kMinWaves = TRACK ? 5 : 7;  // per SIMD: what the kernel reaches by itself  // out = max(1e-10, max_k |x - w|), code = k | sign flag (core/cuda/inf_dist_cuda.cu:131-132,173-177)
     static constexpr int NX = 1, NF = 1, NI = TRACK ? 1 : 0;
     struct State { float best; uint32_t code; };
     __device__ static __forceinline__ void init(State& a) { a.best = kEps; a.code = 0; }
@@ -282,7 +283,10 @@ struct HotInf {  // out = max(1e-10, max_k |x - w|), code = k | sign flag (core/
 };
 
 template <bool TRACK>
-struct HotBound {  // interval bounds (core/cuda/bound_inf_dist_cuda.cu:63,148-151,203-213,225-232)
+struct HotBound {
+    // per SIMD: with the codes the kernel would take 136 registers and run 3; held to 128 (a few cold values spill) it
+    // is 12 % faster
+    static constexpr int kMinWaves = 4;  // interval bounds (core/cuda/bound_inf_dist_cuda.cu:63,148-151,203-213,225-232)
     static constexpr int NX = 2, NF = 2, NI = TRACK ? 2 : 0;
     struct State { float lo, hi; uint32_t wl, wu; };
     __device__ static __forceinline__ void init(State& a) { a.lo = -kEps; a.hi = kEps; a.wl = kNoGradId; a.wu = 0; }
@@ -448,7 +452,7 @@ struct HotOut {
 //   of x; the results turn around in LDS so that every row of the output is written 16 columns at a time.
 // x2off: distance in floats from x (the lower input bound) to the upper one (interval bounds only).
 template <class P>
-__global__ __launch_bounds__(256) void hot_kernel(const float* __restrict__ x, long x2off, const float* __restrict__ w,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(P::kMinWaves))) void hot_kernel(const float* __restrict__ x, long x2off, const float* __restrict__ w,
                                                   const Geom s, const uint32_t* __restrict__ mask_x,
                                                   const uint32_t* __restrict__ mask_w, int nword, int vec, const HotOut out,
                                                   const int* __restrict__ dec, unsigned grid_rows, unsigned grid_cols) {
