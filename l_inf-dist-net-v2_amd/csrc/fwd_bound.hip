@@ -194,8 +194,8 @@ int launch_bound_forward(const float* xl, const float* xu, const float* w, const
         SeedBuffers sb{};
         int rs = launch_row_seeds(xl, w, s, scratch, nullptr, 0, st, &sb, xu, wpre,
                                   hot ? reinterpret_cast<int*>(scratch + nseed) : nullptr);
-        if (!rs && hot) rs = launch_bound_hot(xl, xu, w, s, sb, scratch + nseed, yl, yu, pl, pu, st, &gate);
-        if (!rs && bounded) rs = launch_output_seeds(xl, w, s, sb, gate, 1, st, xu);
+        if (!rs && hot) rs = launch_bound_hot(xl, xu, w, s, sb, scratch + nseed, yl, yu, pl, pu, st, &gate, bounded);
+        if (!rs && bounded && !hot) rs = launch_output_seeds(xl, w, s, sb, gate, 1, st, xu);
         if (rs) {
             (void)scratch_free(scratch, st);
             return rs;

@@ -21,10 +21,12 @@
 // Rounding: the thresholds are evaluated in double with a relative margin of 2^-22, which covers the fp32 rounding
 // of the lower bound and of bx + bw (see hot_threshold).  A row that holds a NaN has a NaN row seed (the pair at its
 // kx may not exist then): all its tiles are hot, and if it is a row of the other side nothing is dead at all.
+#include <algorithm>
 #include <atomic>
 #include <stdlib.h>
 
 #include "ndist_common.h"
+#include "seed_outputs.h"
 
 namespace ndist {
 
@@ -242,6 +244,11 @@ __device__ __forceinline__ bool pair_beats(float ov, uint32_t orank, float v, ui
 
 template <bool TRACK>
 struct HotInf {
+    static constexpr int kSeedLds = kSeedTileFloats;
+    __device__ static __forceinline__ void seed_outputs(const float* x, long, const float* w, const Geom& s,
+                                                        const OutputSeedJob& job, unsigned id, float* lds) {
+        norm_seed_outputs_block(x, w, s, job, id, lds);
+    }
     static constexpr int kMinWaves = TRACK ? 5 : 7;  // per SIMD: what the kernel reaches by itself  // out = max(1e-10, max_k |x - w|), code = k | sign flag (core/cuda/inf_dist_cuda.cu:131-132,173-177)
     static constexpr int NX = 1, NF = 1, NI = TRACK ? 1 : 0;
     struct State { float best; uint32_t code; };
@@ -284,6 +291,11 @@ struct HotInf {
 
 template <bool TRACK>
 struct HotBound {
+    static constexpr int kSeedLds = 2 * kSeedTileFloats;
+    __device__ static __forceinline__ void seed_outputs(const float* x, long x2off, const float* w, const Geom& s,
+                                                        const OutputSeedJob& job, unsigned id, float* lds) {
+        bound_seed_outputs_block(x, x + x2off, w, s, job, id, lds);
+    }
     // per SIMD: with the codes the kernel would take 136 registers and run 3; held to 128 (a few cold values spill) it
     // is 12 % faster
     static constexpr int kMinWaves = 4;  // interval bounds (core/cuda/bound_inf_dist_cuda.cu:63,148-151,203-213,225-232)
@@ -450,16 +462,27 @@ struct HotOut {
 //   dec[0] == 1, the rows of x own: a workgroup takes one row of x and 256 columns (64 per wave).
 //   dec[0] == 2, the rows of w own: a workgroup takes 16 rows of w (four per wave, one after the other) and 64 rows
 //   of x; the results turn around in LDS so that every row of the output is written 16 columns at a time.
+//   dec[0] == 0, the dense kernels queued behind this one run: the first seed_blocks workgroups compute the output
+//   seeds those kernels start from (a launch of its own otherwise; on the hot path every launch that finds itself
+//   gated off costs about as much as the plan kernel's decision saves).
 // x2off: distance in floats from x (the lower input bound) to the upper one (interval bounds only).
 template <class P>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(P::kMinWaves))) void hot_kernel(const float* __restrict__ x, long x2off, const float* __restrict__ w,
                                                   const Geom s, const uint32_t* __restrict__ mask_x,
                                                   const uint32_t* __restrict__ mask_w, int nword, int vec, const HotOut out,
-                                                  const int* __restrict__ dec, unsigned grid_rows, unsigned grid_cols) {
+                                                  const int* __restrict__ dec, unsigned grid_rows, unsigned grid_cols,
+                                                  const OutputSeedJob seeds, unsigned seed_blocks) {
     constexpr int NF = P::NF, NI = P::NI;
-    __shared__ float tv[NF][kHotRows][17];
-    __shared__ uint32_t tc[NI > 0 ? NI : 1][kHotRows][17];
+    // one array for both roles: [NF][kHotRows][17] values and [NI][kHotRows][17] codes, or the tiles of the seeds
+    constexpr int kTurn = (NF + NI) * kHotRows * 17;
+    __shared__ float lds[kTurn > P::kSeedLds ? kTurn : P::kSeedLds];
+    float (*tv)[kHotRows][17] = reinterpret_cast<float (*)[kHotRows][17]>(lds);
+    uint32_t (*tc)[kHotRows][17] = reinterpret_cast<uint32_t (*)[kHotRows][17]>(lds + NF * kHotRows * 17);
     const int choice = dec[0];
+    if (choice == 0) {
+        if (blockIdx.x < seed_blocks) P::seed_outputs(x, x2off, w, s, seeds, blockIdx.x, lds);
+        return;
+    }
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     // the row of the other side whose result this lane ends up with (lanes with (lane & 7) >= kHotSlots: none)
     const int mine = 8 * (lane & 7) + (lane >> 3);
@@ -568,7 +591,7 @@ size_t hot_scratch_floats(const Geom& s) {
 }
 
 static int launch_hot(const float* x, const float* x2, const float* w, const Geom& s, const SeedBuffers& sb, float* base,
-                      const HotOut& out, bool track, hipStream_t st, const int** decision) {
+                      const HotOut& out, bool track, hipStream_t st, const int** decision, bool with_seeds) {
     const int ntile = sb.ntile, nword = ceil_div(ntile, 32), nblk = plan_blocks(s);
     const long rows = (long)s.M * s.G;
     int* dec = reinterpret_cast<int*>(base);  // [0] decision, [1], [2] hot entries per side, [3] ticket (cleared by the row pre-pass)
@@ -586,10 +609,12 @@ static int launch_hot(const float* x, const float* x2, const float* w, const Geo
     const long x2off = x2 != nullptr ? (long)(((intptr_t)x2 - (intptr_t)x) / (intptr_t)sizeof(float)) : 0;
     const unsigned grid_r = (unsigned)(rows * ceil_div(s.COg, 4 * kHotRows));
     const unsigned grid_c = (unsigned)((long)ceil_div(s.M, kHotRows) * ceil_div(s.COg, 16) * s.G);
-    const dim3 grid(grid_r > grid_c ? grid_r : grid_c);
+    const OutputSeedJob job = output_seed_job(s, sb);
+    const unsigned seed_blocks = with_seeds ? (unsigned)((long)job.nmb * job.nnb * s.G) : 0u;
+    const dim3 grid(std::max(std::max(grid_r, grid_c), seed_blocks));
 #define NDIST_HOT(POLICY) \
     hipLaunchKernelGGL(hot_kernel<POLICY>, grid, dim3(256), 0, st, x, x2off, w, s, mask_x, mask_w, nword, vec, out, dec, \
-                       grid_r, grid_c)
+                       grid_r, grid_c, job, seed_blocks)
     if (x2 == nullptr) {
         if (track) NDIST_HOT(HotInf<true>);
         else NDIST_HOT(HotInf<false>);
@@ -602,15 +627,16 @@ static int launch_hot(const float* x, const float* x2, const float* w, const Geo
 }
 
 int launch_inf_hot(const float* x, const float* w, const Geom& s, const SeedBuffers& sb, float* base, float* out,
-                   int32_t* pos, hipStream_t st, const int** decision) {
+                   int32_t* pos, hipStream_t st, const int** decision, bool with_seeds) {
     const HotOut o{{out, nullptr}, {pos, nullptr}};
-    return launch_hot(x, nullptr, w, s, sb, base, o, pos != nullptr, st, decision);
+    return launch_hot(x, nullptr, w, s, sb, base, o, pos != nullptr, st, decision, with_seeds);
 }
 
 int launch_bound_hot(const float* xl, const float* xu, const float* w, const Geom& s, const SeedBuffers& sb, float* base,
-                     float* yl, float* yu, int32_t* pl, int32_t* pu, hipStream_t st, const int** decision) {
+                     float* yl, float* yu, int32_t* pl, int32_t* pu, hipStream_t st, const int** decision,
+                     bool with_seeds) {
     const HotOut o{{yl, yu}, {pl, pu}};
-    return launch_hot(xl, xu, w, s, sb, base, o, pl != nullptr, st, decision);
+    return launch_hot(xl, xu, w, s, sb, base, o, pl != nullptr, st, decision, with_seeds);
 }
 
 }  // namespace ndist

@@ -184,8 +184,9 @@ int launch_inf_forward(const float* x, const float* w, const Geom& s, float* out
         SeedBuffers sb{};
         int rs = launch_row_seeds(x, w, s, scratch, nullptr, 0, st, &sb, nullptr, wpre,
                                   hot ? reinterpret_cast<int*>(scratch + nseed) : nullptr);
-        if (!rs && hot) rs = launch_inf_hot(x, w, s, sb, scratch + nseed, out, pos, st, &gate);
-        if (!rs && bounded) rs = launch_output_seeds(x, w, s, sb, gate, 1, st);
+        // (with the hot-tile kernels ahead, their second launch computes the output seeds when the plan says no)
+        if (!rs && hot) rs = launch_inf_hot(x, w, s, sb, scratch + nseed, out, pos, st, &gate, bounded);
+        if (!rs && bounded && !hot) rs = launch_output_seeds(x, w, s, sb, gate, 1, st);
         if (rs) {
             (void)scratch_free(scratch, st);
             return rs;

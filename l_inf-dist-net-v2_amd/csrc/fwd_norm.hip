@@ -11,6 +11,7 @@
 #include <atomic>
 
 #include "fwd_norm_ops.h"
+#include "seed_outputs.h"
 
 namespace ndist {
 
@@ -287,125 +288,22 @@ __global__ __launch_bounds__(256) void norm_seed_kernel(const SeedSide a, const 
     norm_seed_row(sd, r, ntile);
 }
 
-// Seed of every output: the larger of the two pairs at the k of the row seeds of its x row and of its w row.
-// One workgroup per 64 rows x 64 columns of one group.  The pairs from the x seeds are gathered with the lanes along
-// the rows (a wave then reads inside one row of w), the pairs from the w seeds with the lanes along the columns (inside
-// one row of x), an LDS tile turns the first set around, and the seeds are written with the lanes along the columns.
+// Seed of every output (seed_outputs.h), one workgroup per 64 rows x 64 columns of one group.
 __global__ __launch_bounds__(256) void norm_seed_outputs_kernel(const float* __restrict__ x, const float* __restrict__ w,
-                                                                const Geom s, const float* __restrict__ seed_x,
-                                                                const int32_t* __restrict__ seed_k,
-                                                                const float* __restrict__ seed_w,
-                                                                const int32_t* __restrict__ seed_wk,
-                                                                float* __restrict__ seed, int nmb, int nnb,
+                                                                const Geom s, const OutputSeedJob job,
                                                                 const int* __restrict__ gate, int gate_limit) {
-    __shared__ float tile[64][65];
+    __shared__ float tile[kSeedTileFloats];
     if (gate != nullptr && gate[0] >= gate_limit) return;
-    unsigned id = blockIdx.x;
-    const int nb = (int)(id % (unsigned)nnb);
-    id /= (unsigned)nnb;
-    const int mb = (int)(id % (unsigned)nmb), g = (int)(id / (unsigned)nmb);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int m0 = mb * 64, n0 = nb * 64;
-    {
-        const int m = m0 + lane;
-        float sx = 0.f;
-        int kx = 0;
-        if (m < s.M) {
-            sx = seed_x[(long)m * s.G + g];
-            kx = seed_k[(long)m * s.G + g];
-        }
-#pragma unroll 4
-        for (int c = wave * 16; c < wave * 16 + 16; c++) {
-            const int n = n0 + c;
-            float v = 0.f;
-            if (m < s.M && n < s.COg) v = fabsf(sx - w[w_off(s, g, n, kx)]);
-            tile[lane][c] = v;
-        }
-    }
-    __syncthreads();
-    {
-        const int n = n0 + lane;
-        float sw = 0.f;
-        int kw = 0;
-        if (n < s.COg) {
-            sw = seed_w[g * s.COg + n];
-            kw = seed_wk[g * s.COg + n];
-        }
-#pragma unroll 4
-        for (int rr = wave * 16; rr < wave * 16 + 16; rr++) {
-            const int m = m0 + rr;
-            if (m < s.M && n < s.COg) {
-                const int b = m / s.HW, hw = m - b * s.HW;
-                const float v = fabsf(x[x_off(s, b, g, kw, hw)] - sw);
-                seed[y_off(s, b, g, n, hw)] = fmaxf(fmaxf(tile[rr][lane], v), kEps);
-            }
-        }
-    }
+    norm_seed_outputs_block(x, w, s, job, blockIdx.x, tile);
 }
 
-// The same for the interval bounds: seeds of the upper reduction (max of w - xL, xU - w) and of the lower one (min of
-// the same two) at the k of the row seeds.
 __global__ __launch_bounds__(256) void bound_seed_outputs_kernel(const float* __restrict__ xl, const float* __restrict__ xu,
                                                                  const float* __restrict__ w, const Geom s,
-                                                                 const int32_t* __restrict__ seed_k,
-                                                                 const float* __restrict__ seed_w,
-                                                                 const int32_t* __restrict__ seed_wk,
-                                                                 float* __restrict__ seed_hi, float* __restrict__ seed_lo,
-                                                                 int nmb, int nnb, const int* __restrict__ gate,
+                                                                 const OutputSeedJob job, const int* __restrict__ gate,
                                                                  int gate_limit) {
-    __shared__ float thi[64][65], tlo[64][65];
+    __shared__ float tiles[2 * kSeedTileFloats];
     if (gate != nullptr && gate[0] >= gate_limit) return;
-    unsigned id = blockIdx.x;
-    const int nb = (int)(id % (unsigned)nnb);
-    id /= (unsigned)nnb;
-    const int mb = (int)(id % (unsigned)nmb), g = (int)(id / (unsigned)nmb);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int m0 = mb * 64, n0 = nb * 64;
-    {
-        const int m = m0 + lane;
-        float sl = 0.f, su = 0.f;
-        int kx = 0;
-        if (m < s.M) {
-            kx = seed_k[(long)m * s.G + g];
-            sl = xl[x_off(s, m, g, kx, 0)];
-            su = xu[x_off(s, m, g, kx, 0)];
-            if (sl > su) sl = su = (sl + su) * 0.5f;  // an inverted box collapses to its midpoint, as in the operator
-        }
-#pragma unroll 4
-        for (int c = wave * 16; c < wave * 16 + 16; c++) {
-            const int n = n0 + c;
-            float hi = kEps, lo = -kEps;
-            if (m < s.M && n < s.COg) {
-                const float wv = w[w_off(s, g, n, kx)];
-                const float t1 = wv - sl, t2 = su - wv;
-                hi = fmaxf(t1, t2);
-                lo = fminf(t1, t2);
-            }
-            thi[lane][c] = hi;
-            tlo[lane][c] = lo;
-        }
-    }
-    __syncthreads();
-    {
-        const int n = n0 + lane;
-        float sw = 0.f;
-        int kw = 0;
-        if (n < s.COg) {
-            sw = seed_w[g * s.COg + n];
-            kw = seed_wk[g * s.COg + n];
-        }
-#pragma unroll 4
-        for (int rr = wave * 16; rr < wave * 16 + 16; rr++) {
-            const int m = m0 + rr;
-            if (m < s.M && n < s.COg) {
-                float vl = xl[x_off(s, m, g, kw, 0)], vu = xu[x_off(s, m, g, kw, 0)];
-                if (vl > vu) vl = vu = (vl + vu) * 0.5f;
-                const float t1 = sw - vl, t2 = vu - sw;
-                seed_hi[y_off(s, m, g, n, 0)] = fmaxf(fmaxf(fmaxf(t1, t2), thi[rr][lane]), kEps);
-                seed_lo[y_off(s, m, g, n, 0)] = fminf(fminf(fminf(t1, t2), tlo[rr][lane]), -kEps);
-            }
-        }
-    }
+    bound_seed_outputs_block(xl, xu, w, s, job, blockIdx.x, tiles);
 }
 
 size_t seed_scratch_floats(const Geom& s) {
@@ -485,14 +383,10 @@ int launch_row_seeds(const float* x, const float* w, const Geom& s, float* base,
 
 int launch_output_seeds(const float* x, const float* w, const Geom& s, const SeedBuffers& sb, const int* gate,
                         int gate_limit, hipStream_t st, const float* x2) {
-    const int nmb = ceil_div(s.M, 64), nnb = ceil_div(s.COg, 64);
-    if (x2 == nullptr) {
-        hipLaunchKernelGGL(norm_seed_outputs_kernel, dim3((unsigned)((long)nmb * nnb * s.G)), dim3(256), 0, st, x, w, s,
-                           sb.seed_x, sb.seed_k, sb.seed_w, sb.seed_wk, sb.seed, nmb, nnb, gate, gate_limit);
-    } else {
-        hipLaunchKernelGGL(bound_seed_outputs_kernel, dim3((unsigned)((long)nmb * nnb * s.G)), dim3(256), 0, st, x, x2, w,
-                           s, sb.seed_k, sb.seed_w, sb.seed_wk, sb.seed, sb.seed2, nmb, nnb, gate, gate_limit);
-    }
+    const OutputSeedJob job = output_seed_job(s, sb);
+    const dim3 grid((unsigned)((long)job.nmb * job.nnb * s.G));
+    if (x2 == nullptr) hipLaunchKernelGGL(norm_seed_outputs_kernel, grid, dim3(256), 0, st, x, w, s, job, gate, gate_limit);
+    else hipLaunchKernelGGL(bound_seed_outputs_kernel, grid, dim3(256), 0, st, x, x2, w, s, job, gate, gate_limit);
     return hip_failed(hipGetLastError()) ? 4 : 0;
 }
 

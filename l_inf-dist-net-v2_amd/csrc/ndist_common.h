@@ -154,14 +154,17 @@ int launch_output_seeds(const float* x, const float* w, const Geom& s, const See
 // Mode (ndist_set_hot_mode / NORM_DIST_HOT): -1 the counts decide, 0 off, 1 always the cheaper side, 2 / 3 always the
 // rows of x / of w.
 // `base` starts with the four ints the row pre-pass has to clear (launch_row_seeds' `zero`).
+// with_seeds: when the decision is 0, the last of these launches computes the output seeds in sb.seed (and sb.seed2)
+// that launch_output_seeds would: the caller then does not queue that kernel.
 bool hot_forward_applies(const Geom& s);
 bool hot_alone_applies(const Geom& s);  // fwd_inf.hip: below the size of the seeded kernels, still worth the pre-pass
 size_t hot_scratch_floats(const Geom& s);
 int launch_inf_hot(const float* x, const float* w, const Geom& s, const SeedBuffers& sb, float* base, float* out,
-                   int32_t* pos, hipStream_t st, const int** decision);
+                   int32_t* pos, hipStream_t st, const int** decision, bool with_seeds);
 // the same for the interval bounds (sb from the row pre-pass over both input bounds)
 int launch_bound_hot(const float* xl, const float* xu, const float* w, const Geom& s, const SeedBuffers& sb, float* base,
-                     float* yl, float* yu, int32_t* pl, int32_t* pu, hipStream_t st, const int** decision);
+                     float* yl, float* yu, int32_t* pl, int32_t* pu, hipStream_t st, const int** decision,
+                     bool with_seeds);
 void set_hot_mode(int mode);
 int hot_mode();
 
