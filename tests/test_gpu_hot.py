@@ -149,3 +149,28 @@ def test_decision_follows_the_data(modes):
         got = gpu_bound_forward(xl, xu, w)
         for e, v in zip(expect, got):
             assert np.array_equal(e, v), "interval bounds " + kind
+
+
+@pytest.mark.parametrize("kind", ["normal", "late"])
+def test_long_reductions_where_little_can_be_dropped(modes, kind):
+    """The k-tile skipping kernels on long reductions where they can drop little: dense data, and `late` data that is
+    dense up to three quarters of the k range and has its decisive entries behind that (the thresholds stay loose
+    for most of the walk).  Values and codes are the oracle's (hot tiles off, so that the tiled kernels run)."""
+    modes(0)
+    B, CO, CI = 130, 200, 4096
+    x, w = _data("normal", B, CO, CI, 1, seed=21)
+    if kind == "late":
+        x[:, 3 * CI // 4:, 0] *= 0.05
+        w[:, 3 * CI // 4:] *= 0.05
+        x[np.arange(B), 3 * CI // 4 + np.arange(B), 0] = 9.0
+    eo, ep = O.inf_dist_forward(x, w)
+    out, pos = gpu_inf_forward(x, w)
+    assert np.array_equal(out, eo) and np.array_equal(pos, ep), kind
+    out2, _ = gpu_inf_forward(x, w, with_pos=False)
+    assert np.array_equal(out2, eo), "without codes " + kind
+    xl, xu = _boxes(kind, x, np.random.RandomState(5))
+    expect = O.bound_inf_dist_forward(xl, xu, w)
+    for with_pos in (True, False):
+        got = gpu_bound_forward(xl, xu, w, with_pos=with_pos)
+        for e, v in zip(expect, got):
+            assert v is None or np.array_equal(e, v), "interval bounds " + kind
