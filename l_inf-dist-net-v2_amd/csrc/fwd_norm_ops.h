@@ -278,26 +278,29 @@ struct OpNormSkip {
     template <int TN>
     __device__ static __forceinline__ void row2(Acc (&a)[TN], const FwdParams& P, int, float x0, float,
                                                 const float (&w0)[TN], float x1, float, const float (&w1)[TN]) {
-        float d0[TN], d1[TN], e[TN];
         unsigned long long hot[TN], any = 0;  // wave-wide masks: straight from the compares, no vector round trip
 #pragma unroll
-        for (int j = 0; j < TN; j++) { d0[j] = x0 - w0[j]; d1[j] = x1 - w1[j]; }
-#pragma unroll
         for (int j = 0; j < TN; j++) {
-            e[j] = fmaxf(fabsf(d0[j]), fabsf(d1[j]));
-            hot[j] = __builtin_amdgcn_ballot_w64(e[j] > a[j].t);
+            const float e = fmaxf(fabsf(x0 - w0[j]), fabsf(x1 - w1[j]));
+            hot[j] = __builtin_amdgcn_ballot_w64(e > a[j].t);
             any |= hot[j];
         }
         if (__builtin_expect(any != 0, 0)) {
+            // (the differences are formed again here, from copies the compiler cannot identify with x0 and x1:
+            // kept from above they would occupy 3 * TN registers across the branch and push accumulators into scratch)
+            float xa = x0, xb = x1;
+            asm volatile("" : "+v"(xa), "+v"(xb));
 #pragma unroll
             for (int j = 0; j < TN; j++) {
                 if (hot[j] != 0) {  // some lane has a pair that counts
+                    const float d0 = xa - w0[j], d1 = xb - w1[j];
                     if constexpr (!GIVEN_MAX) {
-                        const float et = e[j] * P.thr;  // above the maximum <=> et above the threshold
-                        if (__builtin_amdgcn_ballot_w64(et > a[j].t) != 0) raise_max(a[j], P, e[j], et);
+                        const float e = fmaxf(fabsf(d0), fabsf(d1));
+                        const float et = e * P.thr;  // above the maximum <=> et above the threshold
+                        if (__builtin_amdgcn_ballot_w64(et > a[j].t) != 0) raise_max(a[j], P, e, et);
                     }
-                    const float e0 = fast_exp2(fmaf(P.p, fast_log2(fabsf(d0[j])), -a[j].c));
-                    const float e1 = fast_exp2(fmaf(P.p, fast_log2(fabsf(d1[j])), -a[j].c));
+                    const float e0 = fast_exp2(fmaf(P.p, fast_log2(fabsf(d0)), -a[j].c));
+                    const float e1 = fast_exp2(fmaf(P.p, fast_log2(fabsf(d1)), -a[j].c));
                     a[j].s += e0;
                     a[j].s += e1;
                 }
