@@ -165,7 +165,8 @@ __global__ __launch_bounds__(256) void bound_rescan_kernel(const float* __restri
 }
 
 int launch_bound_forward(const float* xl, const float* xu, const float* w, const Geom& s, float* yl, float* yu,
-                         int32_t* pl, int32_t* pu, hipStream_t st, const UnfoldGeom* cv, const WeightSeeds* wpre) {
+                         int32_t* pl, int32_t* pu, hipStream_t st, const UnfoldGeom* cv, const WeightSeeds* wpre,
+                         const SharedFront* front) {
     FwdParams P{};
     PatchMap pm{};
     if (cv != nullptr) {
@@ -190,14 +191,22 @@ int launch_bound_forward(const float* xl, const float* xu, const float* w, const
     const int* gate = nullptr;
     if (bounded || hot) {
         const size_t nseed = bound_seed_scratch_floats(s);
-        NDIST_HIP_TRY(scratch_alloc((void**)&scratch, (nseed + (hot ? hot_scratch_floats(s) : 0)) * sizeof(float), st));
         SeedBuffers sb{};
-        int rs = launch_row_seeds(xl, w, s, scratch, nullptr, 0, st, &sb, xu, wpre,
+        int rs = 0;
+        if (front != nullptr) {
+            scratch = front->scratch;
+            sb = front->sb;
+        } else {
+            NDIST_HIP_TRY(scratch_alloc((void**)&scratch, (nseed + (hot ? hot_scratch_floats(s) : 0)) * sizeof(float), st));
+            rs = launch_row_seeds(xl, w, s, scratch, nullptr, 0, st, &sb, xu, wpre,
                                   hot ? reinterpret_cast<int*>(scratch + nseed) : nullptr);
-        if (!rs && hot) rs = launch_bound_hot(xl, xu, w, s, sb, scratch + nseed, yl, yu, pl, pu, st, &gate, bounded);
+        }
+        if (!rs && hot)
+            rs = launch_bound_hot(xl, xu, w, s, sb, scratch + nseed, yl, yu, pl, pu, st, &gate, bounded,
+                                  front != nullptr && front->plan_done);
         if (!rs && bounded && !hot) rs = launch_output_seeds(xl, w, s, sb, gate, 1, st, xu);
         if (rs) {
-            (void)scratch_free(scratch, st);
+            if (front == nullptr) (void)scratch_free(scratch, st);
             return rs;
         }
         if (gate != nullptr) {
@@ -215,7 +224,7 @@ int launch_bound_forward(const float* xl, const float* xu, const float* w, const
     }
     // (the scratch holds the gate: it is released after the last kernel that reads it has been queued)
     auto done = [&](int rc) {
-        if ((bounded || hot) && hip_failed(scratch_free(scratch, st)) && !rc) rc = 4;
+        if ((bounded || hot) && front == nullptr && hip_failed(scratch_free(scratch, st)) && !rc) rc = 4;
         return rc;
     };
     if (pl == nullptr) {
@@ -251,17 +260,28 @@ int launch_bound_forward(const float* xl, const float* xu, const float* w, const
 int launch_inf_bound_forward(const float* x, const float* xl, const float* xu, const float* w, const Geom& s, float* out,
                              int32_t* pos, float* yl, float* yu, int32_t* pl, int32_t* pu, hipStream_t st,
                              const WeightSeeds* cached) {
-    if (cached != nullptr || (!seeded_forward_applies(s) && !(hot_forward_applies(s) && hot_alone_applies(s)))) {
-        // (cached: the caller keeps the pre-pass over w between calls; problems that use none ignore it)
-        const int rc = launch_inf_forward(x, w, s, out, pos, st, nullptr, cached);
-        return rc ? rc : launch_bound_forward(xl, xu, w, s, yl, yu, pl, pu, st, nullptr, cached);
+    const bool bounded = seeded_forward_applies(s);
+    const bool hot = hot_forward_applies(s) && (bounded || hot_alone_applies(s));
+    if (!bounded && !hot) {
+        const int rc = launch_inf_forward(x, w, s, out, pos, st);
+        return rc ? rc : launch_bound_forward(xl, xu, w, s, yl, yu, pl, pu, st);
     }
+    // One row pre-pass for x, the box and (unless the caller keeps them between calls) the weights, one launch of
+    // the hot-tile plan for both operators; each operator's launcher goes on from there with its own scratch.
+    const size_t na = seed_scratch_floats(s), nb = bound_seed_scratch_floats(s);
+    const size_t nh = hot ? hot_scratch_floats(s) : 0;
+    // (both blocks start on a multiple of four floats: the row pre-pass clears four ints at the head of the hot parts)
+    const size_t sa = (na + nh + 3) / 4 * 4, sbz = nb + nh;
     float* block = nullptr;
-    NDIST_HIP_TRY(scratch_alloc((void**)&block, weight_seed_floats(s) * sizeof(float), st));
-    WeightSeeds ws{};
-    int rc = launch_weight_seeds(w, s, block, nullptr, 0, st, &ws);
-    if (!rc) rc = launch_inf_forward(x, w, s, out, pos, st, nullptr, &ws);
-    if (!rc) rc = launch_bound_forward(xl, xu, w, s, yl, yu, pl, pu, st, nullptr, &ws);
+    NDIST_HIP_TRY(scratch_alloc((void**)&block, (sa + sbz) * sizeof(float), st));
+    SharedFront fa{block, SeedBuffers{}, hot}, fb{block + sa, SeedBuffers{}, hot};
+    int rc = launch_joint_row_seeds(x, xl, xu, w, s, fa.scratch, fb.scratch, cached, st, &fa.sb, &fb.sb,
+                                    hot ? reinterpret_cast<int*>(fa.scratch + na) : nullptr,
+                                    hot ? reinterpret_cast<int*>(fb.scratch + nb) : nullptr);
+    if (!rc && hot) rc = launch_joint_hot_plan(s, fa.sb, fa.scratch + na, fb.sb, fb.scratch + nb, st);
+    const WeightSeeds shared{fa.sb.seed_w, fa.sb.seed_wk, fa.sb.tile_w};
+    if (!rc) rc = launch_inf_forward(x, w, s, out, pos, st, nullptr, &shared, &fa);
+    if (!rc) rc = launch_bound_forward(xl, xu, w, s, yl, yu, pl, pu, st, nullptr, &shared, &fb);
     if (hip_failed(scratch_free(block, st)) && !rc) rc = 4;
     return rc;
 }

@@ -84,13 +84,34 @@ __device__ __forceinline__ void hot_group_maxima(const float* __restrict__ seed_
 // Cost of a side = its hot entries x the length of the other side.  mode: 1 always the cheaper side, 2 / 3 always
 // the x / w side, else the cheaper side if it touches at most 1 / frac of all (row, column, tile) triples.
 constexpr int kPlanRows = 64, kPlanRowsPerWave = kPlanRows / 16;
-__global__ __launch_bounds__(1024) void hot_plan_kernel(const float* __restrict__ seed_x, const float* __restrict__ seed_w,
-                                                        const float* __restrict__ tile_x, const float* __restrict__ tile_w,
-                                                        const Geom s, int ntile, int nword, uint32_t* __restrict__ mask_x,
-                                                        uint32_t* __restrict__ mask_w, int* __restrict__ dec,
-                                                        int* __restrict__ partial, int mode, int frac,
-                                                        const float* __restrict__ far_hi,
-                                                        const float* __restrict__ far_lo) {
+// What differs between two plans over the same weights (a layer's distance and its interval bounds in one call): the
+// rows of the first operand with their statistics, and everything the plan writes.
+struct PlanJob {
+    const float* seed_x;
+    const float* tile_x;
+    uint32_t* mask_x;
+    uint32_t* mask_w;
+    int* dec;
+    int* partial;
+    const float* far_hi;  // interval bounds only
+    const float* far_lo;
+};
+// Workgroups [0, nblk) serve job a, [nblk, 2 nblk) job b (launched with nblk workgroups when there is one job).
+__global__ __launch_bounds__(1024) void hot_plan_kernel(const PlanJob ja, const PlanJob jb, int nblk,
+                                                        const float* __restrict__ seed_w,
+                                                        const float* __restrict__ tile_w, const Geom s, int ntile,
+                                                        int nword, int mode, int frac) {
+    const bool second = (int)blockIdx.x >= nblk;
+    const PlanJob& job = second ? jb : ja;
+    const int bid = (int)blockIdx.x - (second ? nblk : 0);
+    const float* __restrict__ seed_x = job.seed_x;
+    const float* __restrict__ tile_x = job.tile_x;
+    uint32_t* __restrict__ mask_x = job.mask_x;
+    uint32_t* __restrict__ mask_w = job.mask_w;
+    int* __restrict__ dec = job.dec;
+    int* __restrict__ partial = job.partial;
+    const float* __restrict__ far_hi = job.far_hi;
+    const float* __restrict__ far_lo = job.far_lo;
     extern __shared__ unsigned sm[];  // 2 * G maxima
     __shared__ int cnt[2];
     __shared__ int is_last;
@@ -109,7 +130,7 @@ __global__ __launch_bounds__(1024) void hot_plan_kernel(const float* __restrict_
     float own[R], fh[R], fl[R];
 #pragma unroll
     for (int i = 0; i < R; i++) {
-        const long r = (long)blockIdx.x * kPlanRows + wave * R + i;
+        const long r = (long)bid * kPlanRows + wave * R + i;
         valid[i] = r < rows + wrows;  // wave-uniform
         isw[i] = r >= rows;
         rr[i] = !valid[i] ? 0 : (isw[i] ? r - rows : r);
@@ -180,17 +201,17 @@ __global__ __launch_bounds__(1024) void hot_plan_kernel(const float* __restrict_
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-        partial[2 * blockIdx.x] = cnt[0];
-        partial[2 * blockIdx.x + 1] = cnt[1];
+        partial[2 * bid] = cnt[0];
+        partial[2 * bid + 1] = cnt[1];
         __threadfence();  // the counts are visible device-wide before the ticket is taken
-        is_last = atomicAdd(&dec[3], 1) == (int)gridDim.x - 1;
+        is_last = atomicAdd(&dec[3], 1) == nblk - 1;
     }
     __syncthreads();
     if (!is_last || wave != 0) return;
     // the last workgroup's first wave adds the counts up (butterfly over the lanes) and decides
     __threadfence();
     long long cx = 0, cw = 0;
-    for (int b = lane; b < (int)gridDim.x; b += 64) {
+    for (int b = lane; b < nblk; b += 64) {
         cx += __atomic_load_n(&partial[2 * b], __ATOMIC_RELAXED);
         cw += __atomic_load_n(&partial[2 * b + 1], __ATOMIC_RELAXED);
     }
@@ -590,20 +611,56 @@ size_t hot_scratch_floats(const Geom& s) {
     return 8 + 2 * (size_t)plan_blocks(s) + (nword + 1) * ((size_t)s.M * s.G + (size_t)s.COg * s.G);
 }
 
+// Where the plan's results lie in an operator's hot scratch (`base`).
+struct HotLayout {
+    int* dec;  // [0] decision, [1], [2] hot entries per side, [3] ticket (cleared by the row pre-pass)
+    int* partial;
+    uint32_t* mask_x;
+    uint32_t* mask_w;
+    int nword, nblk;
+};
+static HotLayout hot_layout(const Geom& s, const SeedBuffers& sb, float* base) {
+    HotLayout h{};
+    h.nword = ceil_div(sb.ntile, 32);
+    h.nblk = plan_blocks(s);
+    h.dec = reinterpret_cast<int*>(base);
+    h.partial = h.dec + 8;
+    h.mask_x = reinterpret_cast<uint32_t*>(h.partial + 2 * h.nblk);
+    h.mask_w = h.mask_x + (long)s.M * s.G * (h.nword + 1);
+    return h;
+}
+static PlanJob plan_job(const HotLayout& h, const SeedBuffers& sb, bool box) {
+    return PlanJob{sb.seed_x, sb.tile_x, h.mask_x, h.mask_w, h.dec, h.partial, box ? sb.far_hi : nullptr,
+                   box ? sb.far_lo : nullptr};
+}
+// at most 1 / 12 of all (row, column, tile) triples: measured at 5120 x 5120 with 512 and with 64 rows, the dense
+// kernels are the faster ones from about a tenth on
+constexpr int kHotFraction = 12;
+
+int launch_joint_hot_plan(const Geom& s, const SeedBuffers& sb, float* base, const SeedBuffers& sb_box, float* base_box,
+                          hipStream_t st) {
+    const HotLayout ha = hot_layout(s, sb, base), hb = hot_layout(s, sb_box, base_box);
+    hipLaunchKernelGGL(hot_plan_kernel, dim3(2 * ha.nblk), dim3(1024), 2 * s.G * sizeof(unsigned), st,
+                       plan_job(ha, sb, false), plan_job(hb, sb_box, true), ha.nblk, sb.seed_w, sb.tile_w, s, sb.ntile,
+                       ha.nword, hot_mode(), kHotFraction);
+    return hip_failed(hipGetLastError()) ? 4 : 0;
+}
+
 static int launch_hot(const float* x, const float* x2, const float* w, const Geom& s, const SeedBuffers& sb, float* base,
-                      const HotOut& out, bool track, hipStream_t st, const int** decision, bool with_seeds) {
-    const int ntile = sb.ntile, nword = ceil_div(ntile, 32), nblk = plan_blocks(s);
+                      const HotOut& out, bool track, hipStream_t st, const int** decision, bool with_seeds,
+                      bool plan_done) {
+    const HotLayout h = hot_layout(s, sb, base);
+    const int nword = h.nword;
     const long rows = (long)s.M * s.G;
-    int* dec = reinterpret_cast<int*>(base);  // [0] decision, [1], [2] hot entries per side, [3] ticket (cleared by the row pre-pass)
-    int* partial = dec + 8;
-    uint32_t* mask_x = reinterpret_cast<uint32_t*>(partial + 2 * nblk);
-    uint32_t* mask_w = mask_x + rows * (nword + 1);
+    int* dec = h.dec;
+    uint32_t* mask_x = h.mask_x;
+    uint32_t* mask_w = h.mask_w;
     *decision = dec;
-    // at most 1 / 12 of all (row, column, tile) triples: measured at 5120 x 5120 with 512 and with 64 rows, the dense
-    // kernels are the faster ones from about a tenth on
-    hipLaunchKernelGGL(hot_plan_kernel, dim3(nblk), dim3(1024), 2 * s.G * sizeof(unsigned), st, sb.seed_x, sb.seed_w,
-                       sb.tile_x, sb.tile_w, s, ntile, nword, mask_x, mask_w, dec, partial, hot_mode(), 12,
-                       x2 != nullptr ? sb.far_hi : nullptr, x2 != nullptr ? sb.far_lo : nullptr);
+    if (!plan_done) {
+        const PlanJob job = plan_job(h, sb, x2 != nullptr);
+        hipLaunchKernelGGL(hot_plan_kernel, dim3(h.nblk), dim3(1024), 2 * s.G * sizeof(unsigned), st, job, job, h.nblk,
+                           sb.seed_w, sb.tile_w, s, sb.ntile, nword, hot_mode(), kHotFraction);
+    }
     int vec = s.CIg % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0;
     if (x2 != nullptr) vec = vec && (uintptr_t)x2 % 16 == 0;
     const long x2off = x2 != nullptr ? (long)(((intptr_t)x2 - (intptr_t)x) / (intptr_t)sizeof(float)) : 0;
@@ -627,16 +684,16 @@ static int launch_hot(const float* x, const float* x2, const float* w, const Geo
 }
 
 int launch_inf_hot(const float* x, const float* w, const Geom& s, const SeedBuffers& sb, float* base, float* out,
-                   int32_t* pos, hipStream_t st, const int** decision, bool with_seeds) {
+                   int32_t* pos, hipStream_t st, const int** decision, bool with_seeds, bool plan_done) {
     const HotOut o{{out, nullptr}, {pos, nullptr}};
-    return launch_hot(x, nullptr, w, s, sb, base, o, pos != nullptr, st, decision, with_seeds);
+    return launch_hot(x, nullptr, w, s, sb, base, o, pos != nullptr, st, decision, with_seeds, plan_done);
 }
 
 int launch_bound_hot(const float* xl, const float* xu, const float* w, const Geom& s, const SeedBuffers& sb, float* base,
                      float* yl, float* yu, int32_t* pl, int32_t* pu, hipStream_t st, const int** decision,
-                     bool with_seeds) {
+                     bool with_seeds, bool plan_done) {
     const HotOut o{{yl, yu}, {pl, pu}};
-    return launch_hot(xl, xu, w, s, sb, base, o, pl != nullptr, st, decision, with_seeds);
+    return launch_hot(xl, xu, w, s, sb, base, o, pl != nullptr, st, decision, with_seeds, plan_done);
 }
 
 }  // namespace ndist

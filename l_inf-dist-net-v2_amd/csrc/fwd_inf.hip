@@ -154,7 +154,7 @@ bool seeded_forward_applies(const Geom& s) {
 }
 
 int launch_inf_forward(const float* x, const float* w, const Geom& s, float* out, int32_t* pos, hipStream_t st,
-                       const UnfoldGeom* cv, const WeightSeeds* wpre) {
+                       const UnfoldGeom* cv, const WeightSeeds* wpre, const SharedFront* front) {
     FwdParams P{};
     P.x = x;
     P.w = w;
@@ -180,15 +180,22 @@ int launch_inf_forward(const float* x, const float* w, const Geom& s, float* out
     KernelTimer timer(st);  // pre-passes + tiled kernel + rescan
     if (bounded || hot) {
         const size_t nseed = seed_scratch_floats(s);
-        NDIST_HIP_TRY(scratch_alloc((void**)&scratch, (nseed + (hot ? hot_scratch_floats(s) : 0)) * sizeof(float), st));
         SeedBuffers sb{};
-        int rs = launch_row_seeds(x, w, s, scratch, nullptr, 0, st, &sb, nullptr, wpre,
+        int rs = 0;
+        if (front != nullptr) {
+            scratch = front->scratch;
+            sb = front->sb;
+        } else {
+            NDIST_HIP_TRY(scratch_alloc((void**)&scratch, (nseed + (hot ? hot_scratch_floats(s) : 0)) * sizeof(float), st));
+            rs = launch_row_seeds(x, w, s, scratch, nullptr, 0, st, &sb, nullptr, wpre,
                                   hot ? reinterpret_cast<int*>(scratch + nseed) : nullptr);
+        }
         // (with the hot-tile kernels ahead, their second launch computes the output seeds when the plan says no)
-        if (!rs && hot) rs = launch_inf_hot(x, w, s, sb, scratch + nseed, out, pos, st, &gate, bounded);
+        if (!rs && hot)
+            rs = launch_inf_hot(x, w, s, sb, scratch + nseed, out, pos, st, &gate, bounded, front != nullptr && front->plan_done);
         if (!rs && bounded && !hot) rs = launch_output_seeds(x, w, s, sb, gate, 1, st);
         if (rs) {
-            (void)scratch_free(scratch, st);
+            if (front == nullptr) (void)scratch_free(scratch, st);
             return rs;
         }
         if (gate != nullptr) {
@@ -205,7 +212,7 @@ int launch_inf_forward(const float* x, const float* w, const Geom& s, float* out
     }
     // (the scratch holds the gate: it is released after the last kernel that reads it has been queued)
     auto done = [&](int rc) {
-        if ((bounded || hot) && hip_failed(scratch_free(scratch, st)) && !rc) rc = 4;
+        if ((bounded || hot) && front == nullptr && hip_failed(scratch_free(scratch, st)) && !rc) rc = 4;
         return rc;
     };
     if (pos == nullptr) {

@@ -274,16 +274,20 @@ __device__ __forceinline__ void norm_seed_row(const SeedSide& sd, long r, int nt
 }
 
 
-// Blocks [0, nblocks_a) serve side a, the others side b (four rows per block).  Does nothing when the probe's count
-// (gate[0]) says that the skipping operator will not run.  `zero`: four ints cleared for the kernels that follow.
-__global__ __launch_bounds__(256) void norm_seed_kernel(const SeedSide a, const SeedSide b, int nblocks_a, int ntile,
+// Blocks [0, nblocks_a) serve side a, the next nblocks_b side b, the others side c (four rows per block).  Does
+// nothing when the probe's count (gate[0]) says that the skipping operator will not run.  `zero`, `zero2`: four ints
+// each, cleared for the kernels that follow.
+__global__ __launch_bounds__(256) void norm_seed_kernel(const SeedSide a, const SeedSide b, const SeedSide c,
+                                                        int nblocks_a, int nblocks_b, int ntile,
                                                         const int* __restrict__ gate, int gate_limit,
-                                                        int* __restrict__ zero) {
+                                                        int* __restrict__ zero, int* __restrict__ zero2) {
     if (zero != nullptr && blockIdx.x == 0 && threadIdx.x < 4) zero[threadIdx.x] = 0;
+    if (zero2 != nullptr && blockIdx.x == 0 && threadIdx.x >= 64 && threadIdx.x < 68) zero2[threadIdx.x - 64] = 0;
     if (gate != nullptr && gate[0] >= gate_limit) return;
-    const bool second = (int)blockIdx.x >= nblocks_a;
-    const SeedSide& sd = second ? b : a;
-    const long r = (long)(blockIdx.x - (second ? nblocks_a : 0)) * 4 + (threadIdx.x >> 6);
+    const int blk = (int)blockIdx.x;
+    const int side = blk < nblocks_a ? 0 : (blk < nblocks_a + nblocks_b ? 1 : 2);
+    const SeedSide& sd = side == 0 ? a : (side == 1 ? b : c);
+    const long r = (long)(blk - (side == 0 ? 0 : (side == 1 ? nblocks_a : nblocks_a + nblocks_b))) * 4 + (threadIdx.x >> 6);
     if (r >= sd.rows) return;  // whole waves leave: the shuffles stay wave-uniform
     norm_seed_row(sd, r, ntile);
 }
@@ -334,16 +338,17 @@ int launch_weight_seeds(const float* w, const Geom& s, float* base, const int* g
     const int ntile = ceil_div(s.CIg, 32);
     *out = weight_seeds_at(base, s);
     const SeedSide sw{w, nullptr, wrows, s.CIg, out->seed_w, out->seed_wk, out->tile_w, nullptr, nullptr};
-    hipLaunchKernelGGL(norm_seed_kernel, dim3((unsigned)((wrows + 3) / 4)), dim3(256), 0, st, sw, SeedSide{}, (int)((wrows + 3) / 4),
-                       ntile, gate, gate_limit, (int*)nullptr);
+    hipLaunchKernelGGL(norm_seed_kernel, dim3((unsigned)((wrows + 3) / 4)), dim3(256), 0, st, sw, SeedSide{}, SeedSide{},
+                       (int)((wrows + 3) / 4), 0, ntile, gate, gate_limit, (int*)nullptr, (int*)nullptr);
     return hip_failed(hipGetLastError()) ? 4 : 0;
 }
 
-int launch_row_seeds(const float* x, const float* w, const Geom& s, float* base, const int* gate, int gate_limit,
-                     hipStream_t st, SeedBuffers* out, const float* x2, const WeightSeeds* wpre, int* zero) {
+// Where the results of the row pre-pass lie in an operator's seed scratch (`base`), and the two sides of its launch:
+// the rows of x (of the box when x2 is given) and, unless `wpre` brings them, the rows of w.
+static void layout_row_seeds(const float* x, const float* w, const Geom& s, float* base, const float* x2,
+                             const WeightSeeds* wpre, SeedBuffers* out, SeedSide* side_x, SeedSide* side_w) {
     const long rows = (long)s.M * s.G, wrows = (long)s.COg * s.G, total = (long)s.M * s.COg * s.G;
     const int ntile = ceil_div(s.CIg, 32);
-    int rc = 0;
     float* seed_x = base;
     int32_t* seed_k = reinterpret_cast<int32_t*>(seed_x + rows);
     float* seed_w = reinterpret_cast<float*>(seed_k + rows);
@@ -357,16 +362,11 @@ int launch_row_seeds(const float* x, const float* w, const Geom& s, float* base,
         seed_wk = wpre->seed_wk;
         tile_w = wpre->tile_w;
     }
-    // one launch for the rows of x and (unless done before) the rows of w
     // (interval bounds: the two extra row statistics lie behind the second seed array)
     float* far_hi = x2 != nullptr ? after_tiles + total : nullptr;
     float* far_lo = x2 != nullptr ? far_hi + rows : nullptr;
-    const SeedSide sx{x, x2, rows, s.CIg, seed_x, seed_k, tile_x, far_hi, far_lo};
-    const SeedSide sw{w, nullptr, wpre != nullptr ? 0 : wrows, s.CIg, seed_w, seed_wk, tile_w, nullptr, nullptr};
-    const int nbx = (int)((rows + 3) / 4), nbw = (int)((sw.rows + 3) / 4);
-    hipLaunchKernelGGL(norm_seed_kernel, dim3((unsigned)(nbx + nbw)), dim3(256), 0, st, sx, sw, nbx, ntile, gate, gate_limit,
-                       zero);
-    if (hip_failed(hipGetLastError())) rc = 4;
+    *side_x = SeedSide{x, x2, rows, s.CIg, seed_x, seed_k, tile_x, far_hi, far_lo};
+    *side_w = SeedSide{w, nullptr, wpre != nullptr ? 0 : wrows, s.CIg, seed_w, seed_wk, tile_w, nullptr, nullptr};
     out->seed = seed;
     out->seed2 = x2 != nullptr ? after_tiles : nullptr;  // interval bounds: the second seed array lies behind the tile bounds
     out->tile_x = tile_x;
@@ -378,7 +378,32 @@ int launch_row_seeds(const float* x, const float* w, const Geom& s, float* base,
     out->seed_k = seed_k;
     out->seed_w = seed_w;
     out->seed_wk = seed_wk;
-    return rc;
+}
+
+int launch_row_seeds(const float* x, const float* w, const Geom& s, float* base, const int* gate, int gate_limit,
+                     hipStream_t st, SeedBuffers* out, const float* x2, const WeightSeeds* wpre, int* zero) {
+    SeedSide sx{}, sw{};
+    layout_row_seeds(x, w, s, base, x2, wpre, out, &sx, &sw);
+    // one launch for the rows of x and (unless done before) the rows of w
+    const int nbx = (int)((sx.rows + 3) / 4), nbw = (int)((sw.rows + 3) / 4);
+    hipLaunchKernelGGL(norm_seed_kernel, dim3((unsigned)(nbx + nbw)), dim3(256), 0, st, sx, sw, SeedSide{}, nbx, nbw,
+                       out->ntile, gate, gate_limit, zero, (int*)nullptr);
+    return hip_failed(hipGetLastError()) ? 4 : 0;
+}
+
+// The row pre-passes of a layer's distance (x) and of its interval bounds (the box xl, xu) in one launch, with the
+// rows of w unless `wpre` brings them; both operators then read the same results for w.
+int launch_joint_row_seeds(const float* x, const float* xl, const float* xu, const float* w, const Geom& s, float* base,
+                           float* base_box, const WeightSeeds* wpre, hipStream_t st, SeedBuffers* out,
+                           SeedBuffers* out_box, int* zero, int* zero_box) {
+    SeedSide sx{}, sw{}, sb{}, unused{};
+    layout_row_seeds(x, w, s, base, nullptr, wpre, out, &sx, &sw);
+    const WeightSeeds shared{out->seed_w, out->seed_wk, out->tile_w};  // wherever the first layout put (or found) them
+    layout_row_seeds(xl, w, s, base_box, xu, &shared, out_box, &sb, &unused);
+    const int nbx = (int)((sx.rows + 3) / 4), nbb = (int)((sb.rows + 3) / 4), nbw = (int)((sw.rows + 3) / 4);
+    hipLaunchKernelGGL(norm_seed_kernel, dim3((unsigned)(nbx + nbb + nbw)), dim3(256), 0, st, sx, sb, sw, nbx, nbb,
+                       out->ntile, (const int*)nullptr, 0, zero, zero_box);
+    return hip_failed(hipGetLastError()) ? 4 : 0;
 }
 
 int launch_output_seeds(const float* x, const float* w, const Geom& s, const SeedBuffers& sb, const int* gate,

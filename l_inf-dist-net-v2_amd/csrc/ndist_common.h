@@ -146,6 +146,18 @@ int launch_row_seeds(const float* x, const float* w, const Geom& s, float* base,
                      int* zero = nullptr);
 int launch_output_seeds(const float* x, const float* w, const Geom& s, const SeedBuffers& sb, const int* gate,
                         int gate_limit, hipStream_t st, const float* x2 = nullptr);
+// The row kernels of a layer's distance (x into `base`) and of its interval bounds (the box xl, xu into `base_box`)
+// in one launch, with the rows of w unless `wpre` brings them; `zero`, `zero_box`: as `zero` above, one per operator.
+int launch_joint_row_seeds(const float* x, const float* xl, const float* xu, const float* w, const Geom& s, float* base,
+                           float* base_box, const WeightSeeds* wpre, hipStream_t st, SeedBuffers* out,
+                           SeedBuffers* out_box, int* zero, int* zero_box);
+// What the caller of a joint call has queued for one of its two operators before the operator's own launcher runs:
+// scratch (owned by the caller), the results of the row pre-pass, and whether the hot-tile plan is among it.
+struct SharedFront {
+    float* scratch;
+    SeedBuffers sb;
+    bool plan_done;
+};
 
 // p = inf forward through hot k-tiles (fwd_hot.hip).  Queues the kernels that decide, from the row seeds and tile
 // bounds in `sb`, whether few enough k-tiles can hold the maxima, and the kernels that then compute out (and pos
@@ -156,15 +168,18 @@ int launch_output_seeds(const float* x, const float* w, const Geom& s, const See
 // `base` starts with the four ints the row pre-pass has to clear (launch_row_seeds' `zero`).
 // with_seeds: when the decision is 0, the last of these launches computes the output seeds in sb.seed (and sb.seed2)
 // that launch_output_seeds would: the caller then does not queue that kernel.
+// plan_done: the deciding kernel has been queued already (launch_joint_hot_plan, for both operators of a joint call).
 bool hot_forward_applies(const Geom& s);
 bool hot_alone_applies(const Geom& s);  // fwd_inf.hip: below the size of the seeded kernels, still worth the pre-pass
 size_t hot_scratch_floats(const Geom& s);
 int launch_inf_hot(const float* x, const float* w, const Geom& s, const SeedBuffers& sb, float* base, float* out,
-                   int32_t* pos, hipStream_t st, const int** decision, bool with_seeds);
+                   int32_t* pos, hipStream_t st, const int** decision, bool with_seeds, bool plan_done = false);
 // the same for the interval bounds (sb from the row pre-pass over both input bounds)
 int launch_bound_hot(const float* xl, const float* xu, const float* w, const Geom& s, const SeedBuffers& sb, float* base,
                      float* yl, float* yu, int32_t* pl, int32_t* pu, hipStream_t st, const int** decision,
-                     bool with_seeds);
+                     bool with_seeds, bool plan_done = false);
+int launch_joint_hot_plan(const Geom& s, const SeedBuffers& sb, float* base, const SeedBuffers& sb_box, float* base_box,
+                          hipStream_t st);
 void set_hot_mode(int mode);
 int hot_mode();
 
@@ -266,11 +281,14 @@ bool patch_rows_applies(const UnfoldGeom& u);
 int launch_fold_rows(const float* g, const UnfoldGeom& u, float* gx, hipStream_t st);
 // The forward launchers take an optional patch geometry `cv`: x (xl, xu) are then images [B, C, H, W], s describes
 // the unfolded problem (CIg = C / G * kh * kw, HW = OH * OW) and the kernels extract the patches while loading.
+// `front`: the row pre-pass (and the hot-tile plan) of this call are queued already, by launch_inf_bound_forward
 int launch_inf_forward(const float* x, const float* w, const Geom& s, float* out, int32_t* pos, hipStream_t st,
-                       const UnfoldGeom* cv = nullptr, const WeightSeeds* wpre = nullptr);
+                       const UnfoldGeom* cv = nullptr, const WeightSeeds* wpre = nullptr,
+                       const SharedFront* front = nullptr);
 int launch_bound_forward(const float* xl, const float* xu, const float* w, const Geom& s,
                          float* yl, float* yu, int32_t* pl, int32_t* pu, hipStream_t st,
-                         const UnfoldGeom* cv = nullptr, const WeightSeeds* wpre = nullptr);
+                         const UnfoldGeom* cv = nullptr, const WeightSeeds* wpre = nullptr,
+                         const SharedFront* front = nullptr);
 // true when the two launchers above would run their seeded (k-tile skipping) variants on this problem
 bool seeded_forward_applies(const Geom& s);
 // the distance of x and the interval bounds of (xl, xu) against the same weights, pre-passes over w shared
