@@ -32,10 +32,15 @@ _ext = None
 EXTENSION_PATH = os.path.join(os.path.dirname(_LIB_PATH), "norm_dist_hip_ext.so")
 if os.environ.get("NORM_DIST_BINDING", "ext") != "ctypes" and os.path.exists(EXTENSION_PATH):
     import importlib.util
-    _spec = importlib.util.spec_from_file_location("norm_dist_hip_ext", EXTENSION_PATH)
-    _ext = importlib.util.module_from_spec(_spec)
-    _spec.loader.exec_module(_ext)
-    sys.modules.setdefault("norm_dist_hip_ext", _ext)
+    try:
+        _spec = importlib.util.spec_from_file_location("norm_dist_hip_ext", EXTENSION_PATH)
+        _ext = importlib.util.module_from_spec(_spec)
+        _spec.loader.exec_module(_ext)
+        sys.modules.setdefault("norm_dist_hip_ext", _ext)
+    except ImportError as _exc:  # built against another torch: the ctypes route serves the same C ABI
+        import warnings
+        warnings.warn("norm_dist_hip_ext could not be loaded (%s); using the ctypes binding" % _exc)
+        _ext = None
 BINDING = "ext" if _ext is not None else "ctypes"
 
 _P = ctypes.c_void_p

@@ -29,10 +29,36 @@ class NormDistBase(nn.Module):
         self.tag = NormDistBase.tag
         self._weight_cache = WeightCache()  # plain attribute: not a parameter or buffer, never in the state dict
 
+    def freeze_weights(self):
+        """Opt in to keeping the p = inf forwards' pre-pass over the weights between calls (evaluation,
+        certification, serving; no counterpart in the reference).  Takes the pre-pass now; from here on the caller
+        promises that the weights keep their values until `unfreeze_weights()`.  `train()`, `load_state_dict` and
+        moves between devices unfreeze; in-place updates that advance the parameter's version counter redo the
+        pre-pass; writes through `weight.data` are invisible to torch: call `freeze_weights()` again after them.
+        Returns True when the weights could be cached (contiguous float32 on the GPU)."""
+        return self._weight_cache.freeze(self.weight, self.groups)
+
+    def unfreeze_weights(self):
+        self._weight_cache.drop()
+
+    def train(self, mode=True):
+        if mode:
+            self._weight_cache.drop()
+        return super().train(mode)
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        self._weight_cache.drop()
+        return super()._load_from_state_dict(*args, **kwargs)
+
+    def _apply(self, fn, *args, **kwargs):
+        self._weight_cache.drop()
+        return super()._apply(fn, *args, **kwargs)
+
     def forward(self, x=None, lower=None, upper=None):
-        # evaluation without gradients: the weights stand still from call to call, their pre-pass is kept
-        frozen = not self.training and not torch.is_grad_enabled() and math.isinf(self.p) and self.weight.is_cuda
-        cache = self._weight_cache if frozen else None
+        # kept pre-pass of the weights: only after freeze_weights(), only in evaluation without gradients
+        use = (self._weight_cache.frozen and not self.training and not torch.is_grad_enabled() and math.isinf(self.p)
+               and self.weight.is_cuda)
+        cache = self._weight_cache if use else None
         if x is not None and lower is not None and upper is not None and math.isinf(self.p) and x.is_cuda:
             # the distance and its bounds against the same weights: one call (shares the pre-pass over the weights)
             x, lower, upper = inf_dist_with_bounds(x, lower, upper, self.weight, self.groups, tag=self.tag, cache=cache)
@@ -62,6 +88,17 @@ class NormDistBase(nn.Module):
             b = self.bias.view(1, -1, 1)
             x, lower, upper = apply_if_not_none((x, lower, upper), lambda t: t + b)
         return x, lower, upper
+
+
+def freeze_weights(model):
+    """`freeze_weights()` on every distance layer of `model`; returns how many layers now keep their pre-pass."""
+    return sum(bool(m.freeze_weights()) for m in model.modules() if isinstance(m, NormDistBase))
+
+
+def unfreeze_weights(model):
+    for m in model.modules():
+        if isinstance(m, NormDistBase):
+            m.unfreeze_weights()
 
 
 class NormDistConv(NormDistBase):

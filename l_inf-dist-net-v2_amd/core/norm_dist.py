@@ -289,29 +289,53 @@ def conv_bound_inf_dist(x_lower, x_upper, weight, kernel_size, dilation=1, paddi
 
 
 class WeightCache:
-    """The p = inf forwards' pre-pass over a layer's weights, kept while the weights stay as they are (evaluation,
-    certification, serving) and redone when they change: the key is the parameter's storage address and version
-    counter, which every in-place update (optimizer step, load_state_dict, copy_) advances.  No counterpart in the
-    reference."""
+    """The p = inf forwards' pre-pass over a layer's weights, taken once by `freeze(weight, groups)` and handed to the
+    *_cached entry points until `drop()`.  Strictly opt-in (the layers' `freeze_weights()`): while frozen the caller
+    promises that the weights keep their values.  Updates that torch can see (a new parameter tensor, another
+    storage address, an advanced version counter, another shape or device) still redo the pre-pass, but writes
+    through `weight.data` advance no counter and cannot be seen: after such a write call `freeze` again or `drop`.
+    Non-contiguous weights are never cached (their contiguous copy is a new tensor on every call).  No counterpart
+    in the reference, which keeps no state between calls."""
 
     def __init__(self):
-        self._key, self._buffer = None, None
+        self._key, self._buffer, self.frozen = None, None, False
+
+    @staticmethod
+    def _key_of(weight, groups):
+        return (weight.data_ptr(), weight._version, tuple(weight.shape), groups, weight.device)
+
+    def freeze(self, weight, groups):
+        """Take (or retake) the pre-pass of `weight` as it is now."""
+        self.drop()
+        if weight.is_cuda and weight.dtype == torch.float32 and weight.is_contiguous():
+            self._buffer = _C.weight_cache(weight.detach(), groups)
+            self._key = self._key_of(weight, groups)
+            self.frozen = True
+        return self.frozen
+
+    def drop(self):
+        self._key, self._buffer, self.frozen = None, None, False
 
     def get(self, weight, groups):
-        key = (weight.data_ptr(), weight._version, tuple(weight.shape), groups, weight.device)
-        if key != self._key:
-            self._buffer = _C.weight_cache(weight.detach().contiguous(), groups)
-            self._key = key
+        """The kept buffer for `weight`, retaken when torch shows that the weights changed; None when not frozen or
+        when `weight` cannot be cached."""
+        if not self.frozen:
+            return None
+        if not (weight.is_cuda and weight.is_contiguous()):
+            return None
+        if self._key_of(weight, groups) != self._key:
+            self.freeze(weight, groups)
         return self._buffer
 
 
 def inf_dist_nograd(x, weight, groups=1, cache=None):
     """The infinity distance without gradients, optionally with the weights' pre-pass taken from `cache`
     (WeightCache)."""
+    buffer = cache.get(weight, groups) if cache is not None else None
     x, weight = x.contiguous(), weight.contiguous()
     y = _new_output(x, weight)
-    if cache is not None:
-        _C.inf_dist_forward_nograd_cached(x, weight, cache.get(weight, groups), y, groups)
+    if buffer is not None:
+        _C.inf_dist_forward_nograd_cached(x, weight, buffer, y, groups)
     else:
         _C.inf_dist_forward_nograd(x, weight, y, groups)
     return y
@@ -325,12 +349,12 @@ def inf_dist_with_bounds(x, x_lower, x_upper, weight, groups=1, tag=None, cache=
     tensors = (x, x_lower, x_upper, weight)
     if (all(t.is_cuda and t.dtype == torch.float32 for t in tensors)
             and not (torch.is_grad_enabled() and any(t.requires_grad for t in tensors))):
+        buffer = cache.get(weight, groups) if cache is not None else None
         x, x_lower, x_upper, weight = (t.contiguous() for t in tensors)
         y = _new_output(x, weight)
         y_lower, y_upper = torch.empty_like(y), torch.empty_like(y)
-        if cache is not None:
-            _C.inf_and_bound_forward_nograd_cached(x, x_lower, x_upper, weight, cache.get(weight, groups), y, y_lower,
-                                                   y_upper, groups)
+        if buffer is not None:
+            _C.inf_and_bound_forward_nograd_cached(x, x_lower, x_upper, weight, buffer, y, y_lower, y_upper, groups)
         else:
             _C.inf_and_bound_forward_nograd(x, x_lower, x_upper, weight, y, y_lower, y_upper, groups)
         return y, y_lower, y_upper

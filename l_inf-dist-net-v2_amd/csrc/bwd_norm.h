@@ -48,7 +48,9 @@ struct BwdParams {
     // second gate of the same form: chooses between the two skipping variants (term by term, or by bounds first)
     const int* gate2;
     int gate2_limit, gate2_sense;
-    long g_off;       // unfolded variant only: offset in floats from the 1/out factors to the grad_output factors
+    long g_off;       // offset in floats from the factors to a second array of the same layout, 0 if there is none:
+                      // grad_output (IP -2, whose factors are 1/out), or the part of every factor that float32
+                      // dropped (IP -5, and the rare branch of the skipping variants -3 / -4)
     // Reproducible grad_input (row-split kernel): a workgroup that holds ALL units of a (group, slab, row chunk) block
     // stores that block's grad_input directly; a block shared between neighbouring workgroups goes into `part`
     // ([workgroup][2][rows per workgroup][64]: slot 0 for the block a workgroup starts in, slot 1 for the one it ends
@@ -65,18 +67,31 @@ __device__ __forceinline__ f16v load_factors(const float* p) {
     typedef const f16v __attribute__((address_space(4))) * cptr;
     return *reinterpret_cast<cptr>(reinterpret_cast<uintptr_t>(p));
 }
+// one factor through the scalar data cache (wave-uniform address)
+__device__ __forceinline__ float load_factor(const float* p) {
+    typedef const float __attribute__((address_space(4))) * cptr;
+    return *reinterpret_cast<cptr>(reinterpret_cast<uintptr_t>(p));
+}
 constexpr int kBwdRowBatch = 16;  // rows whose factors are fetched by one 16-dword scalar load
 
 // one (row, co, ci) term for a row slot of the lane, given the wave-uniform factor of that (row, co)
 // R terms (R consecutive row slots of the lane, one co) given the wave-uniform factors of those (row, co) pairs.
 // IP: 0..8 the exponent p-1 by repeated multiplication; -1 / -3 general exponent >= 1 (grad_output folded into the
 // factor); -2 general exponent < 1, where the root that folds grad_output could overflow: `a` is 1/out and
-// grad_output comes separately in `g2`.
+// grad_output comes separately in `g2`; -5 general exponent >= 1 with a compensated product (large exponents): `g2`
+// is the part of the factor that float32 dropped.
+// Large exponents multiply every rounding under the power by q = p - 1: with v = fl(t * a) and a = fl(a_exact) the
+// term carries q * (two roundings) on top of the rounding of t = x - w that no float32 evaluation avoids, which at
+// q = 200 is 1 - 2e-5 relative against the 1e-5 the operator is held to.  Both are known exactly:
+// e = fma(t, a, -v) + t * a_lo is what v is missing (a_lo from the pre-pass, which forms the factor in double
+// precision), and sign(v + e)|v + e|^q = |v|^(q-1) * (v + q e) to first order: three more instructions, used from
+// q = 24 on (-5) and in the rare branch of the skipping variants (`lo` != nullptr).
 // The arithmetic is laid out in stages over the R rows: back-to-back dependent vector instructions stall a wave,
 // independent neighbours do not.
 template <int IP, bool WITH_W, int R>
 __device__ __forceinline__ void bwd_terms(const float* __restrict__ xv, float wv, const float (&a)[R], const float (&g2)[R],
-                                          float q, float thr, float* __restrict__ gxa, float (&gwp)[R]) {
+                                          float q, float thr, float* __restrict__ gxa, float (&gwp)[R],
+                                          const float* __restrict__ lo = nullptr) {
     float t[R];
 #pragma unroll
     for (int r = 0; r < R; r++) t[r] = xv[r] - wv;
@@ -123,10 +138,40 @@ __device__ __forceinline__ void bwd_terms(const float* __restrict__ xv, float wv
             for (int r = 0; r < R; r++) {
                 if (hot[r] != 0) {
                     const float e = fast_exp2(q1 * fast_log2(fabsf(t[r])));
-                    gxa[r] = fmaf(t[r], e, gxa[r]);
-                    if (WITH_W) gwp[r] = fmaf(t[r], e, gwp[r]);
+                    float v = t[r];
+                    if (lo != nullptr) {
+                        // what v = fl((x - w) * a) is missing of (x - w) * a_exact; a_lo of this row through the
+                        // scalar cache, only here (wave-uniform address)
+                        const float d = xv[r] - wv;
+                        const float miss = fmaf(d, load_factor(lo + r), fmaf(d, a[r], -v));
+                        v = fmaf(q, miss, v);
+                    }
+                    gxa[r] = fmaf(v, e, gxa[r]);
+                    if (WITH_W) gwp[r] = fmaf(v, e, gwp[r]);
                 }
             }
+        }
+    } else if constexpr (IP == -5) {
+        // IP -1 with the compensated product: g2 = a_lo
+        float e[R], v[R], miss[R];
+        const float q1 = q - 1.0f;
+#pragma unroll
+        for (int r = 0; r < R; r++) v[r] = t[r] * a[r];
+#pragma unroll
+        for (int r = 0; r < R; r++) miss[r] = fmaf(t[r], a[r], -v[r]);
+#pragma unroll
+        for (int r = 0; r < R; r++) e[r] = fast_log2(fabsf(v[r]));
+#pragma unroll
+        for (int r = 0; r < R; r++) miss[r] = fmaf(t[r], g2[r], miss[r]);
+#pragma unroll
+        for (int r = 0; r < R; r++) e[r] = fast_exp2(q1 * e[r]);
+#pragma unroll
+        for (int r = 0; r < R; r++) v[r] = fmaf(q, miss[r], v[r]);
+#pragma unroll
+        for (int r = 0; r < R; r++) gxa[r] = fmaf(v[r], e[r], gxa[r]);
+        if (WITH_W) {
+#pragma unroll
+            for (int r = 0; r < R; r++) gwp[r] = fmaf(v[r], e[r], gwp[r]);
         }
     } else if constexpr (IP == -1) {
         // general exponent q >= 1: sign(v)|v|^q = v * |v|^(q-1), the power through the hardware exp2 / log2 and the
@@ -334,7 +379,7 @@ __global__ __launch_bounds__(64 * NW, 4) void bwd_fused_kernel(const float* __re
     const float* __restrict__ ap = factor_ptr(cur);
     f16v a_cur = load_factors(ap);
     f16v g_cur = a_cur;
-    if constexpr (IP == -2) g_cur = load_factors(ap + P.g_off);
+    if constexpr (IP == -2 || IP == -5) g_cur = load_factors(ap + P.g_off);
     {
         float w0[WPT];
         fetch_w(cur, w0);
@@ -415,7 +460,8 @@ __global__ __launch_bounds__(64 * NW, 4) void bwd_fused_kernel(const float* __re
 #pragma unroll
                         for (int r = 0; r < 4; r++)
                             ga[r] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(av), lane0 + q0 + r));
-                        bwd_terms<-3, WITH_W, 4>(&xv[q0], wv, ga, ga, P.q, thr, &gxa[q0], gwp);
+                        bwd_terms<-3, WITH_W, 4>(&xv[q0], wv, ga, ga, P.q, thr, &gxa[q0], gwp,
+                                                 P.g_off != 0 ? arow + P.g_off + (long)cl * P.Mpad + q0 : nullptr);
                     }
                 }
                 if (WITH_W) {
@@ -473,7 +519,8 @@ __global__ __launch_bounds__(64 * NW, 4) void bwd_fused_kernel(const float* __re
                     float ga[RG], gg[RG];
 #pragma unroll
                     for (int r = 0; r < RG; r++) { ga[r] = fa[q0 + r]; gg[r] = fg[q0 + r]; }
-                    bwd_terms<IP, WITH_W, RG>(&xv[bi * RB + q0], wv, ga, gg, P.q, thr, &gxa[bi * RB + q0], gwp);
+                    bwd_terms<IP, WITH_W, RG>(&xv[bi * RB + q0], wv, ga, gg, P.q, thr, &gxa[bi * RB + q0], gwp,
+                                              IP == -3 && P.g_off != 0 ? ap + P.g_off + q0 : nullptr);
                 };
                 // first rows of the batch: their use of the factors is where the wait for the pending request lands
                 group(0);
@@ -485,7 +532,7 @@ __global__ __launch_bounds__(64 * NW, 4) void bwd_fused_kernel(const float* __re
                     bi + 1 < NB ? ap + RB : (last_co ? ap_next_unit : ap + (P.Mpad - (NB - 1) * RB));
                 const f16v a_nxt = load_factors(apn);
                 f16v g_nxt = a_nxt;
-                if constexpr (IP == -2) g_nxt = load_factors(apn + P.g_off);
+                if constexpr (IP == -2 || IP == -5) g_nxt = load_factors(apn + P.g_off);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int q0 = RG; q0 < RB; q0 += RG) group(q0);
@@ -575,7 +622,7 @@ __global__ __launch_bounds__(64 * kBwdSmallWaves) void bwd_small_kernel(const fl
     const float* __restrict__ wp = W + w_off(s, g, co_begin, cic);
     f16v a_cur = load_factors(ap);
     f16v g_cur = a_cur;
-    if constexpr (IP == -2) g_cur = load_factors(ap + P.g_off);
+    if constexpr (IP == -2 || IP == -5) g_cur = load_factors(ap + P.g_off);
     float wnext = *wp;
     for (int co = co_begin; co < co_end; co++) {
         const float wv = wnext;
@@ -592,7 +639,8 @@ __global__ __launch_bounds__(64 * kBwdSmallWaves) void bwd_small_kernel(const fl
                 float ga[RG], gg[RG];
 #pragma unroll
                 for (int r = 0; r < RG; r++) { ga[r] = fa[q0 + r]; gg[r] = fg[q0 + r]; }
-                bwd_terms<IP, WITH_W, RG>(&xv[bi * RB + q0], wv, ga, gg, P.q, thr, &gxa[bi * RB + q0], gwp);
+                bwd_terms<IP, WITH_W, RG>(&xv[bi * RB + q0], wv, ga, gg, P.q, thr, &gxa[bi * RB + q0], gwp,
+                                          IP == -3 && P.g_off != 0 ? ap + P.g_off + q0 : nullptr);
             };
             group(0);
             __builtin_amdgcn_sched_barrier(0);
@@ -600,7 +648,7 @@ __global__ __launch_bounds__(64 * kBwdSmallWaves) void bwd_small_kernel(const fl
             const float* __restrict__ apn = bi + 1 < NB ? ap + RB : (last_co ? ap - (NB - 1) * RB : ap + (P.Mpad - (NB - 1) * RB));
             const f16v a_nxt = load_factors(apn);
             f16v g_nxt = a_nxt;
-            if constexpr (IP == -2) g_nxt = load_factors(apn + P.g_off);
+            if constexpr (IP == -2 || IP == -5) g_nxt = load_factors(apn + P.g_off);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int q0 = RG; q0 < RB; q0 += RG) group(q0);

@@ -10,6 +10,7 @@ template <> int launch_bwd_ip<7>(const BwdPtrs& a, const BwdParams& P, int cfg, 
 template <> int launch_bwd_ip<-1>(const BwdPtrs& a, const BwdParams& P, int cfg, int grid, hipStream_t st) { return launch_bwd_ip_impl<-1>(a, P, cfg, grid, st); }
 template <> int launch_bwd_ip<-3>(const BwdPtrs& a, const BwdParams& P, int cfg, int grid, hipStream_t st) { return launch_bwd_ip_impl<-3>(a, P, cfg, grid, st); }
 template <> int launch_bwd_ip<-2>(const BwdPtrs& a, const BwdParams& P, int cfg, int grid, hipStream_t st) { return launch_bwd_ip_impl<-2>(a, P, cfg, grid, st); }
+template <> int launch_bwd_ip<-5>(const BwdPtrs& a, const BwdParams& P, int cfg, int grid, hipStream_t st) { return launch_bwd_ip_impl<-5>(a, P, cfg, grid, st); }
 // skipping by bounds (row-split configurations only)
 template <> int launch_bwd_ip<-4>(const BwdPtrs& a, const BwdParams& P, int cfg, int grid, hipStream_t st) {
     if (cfg > 2) return 2;  // not instantiated for the small-batch kernel
@@ -90,11 +91,12 @@ __global__ __launch_bounds__(256) void bwd_gx_fixup_kernel(const float* __restri
 
 // pre-pass: the per-(row, co) factor, transposed to [gco][m]
 //   p = 1: grad_output ;  p >= 2: sign(g) * |g|^(1/(p-1)) / out  (root in double precision: its error is multiplied
-//   by p-1 when the main kernel raises the factor to that power again) ;  1 < p < 2 (g_off != 0): 1/out, and
-//   grad_output in a second array g_off floats further
+//   by p-1 when the main kernel raises the factor to that power again) ;  1 < p < 2 (second == 1): 1/out, and
+//   grad_output in a second array g_off floats further ;  second == 2 (large exponents): the second array holds
+//   what the float32 factor dropped of the double-precision one
 __global__ __launch_bounds__(256) void bwd_prepare_kernel(const float* __restrict__ out, const float* __restrict__ gout,
                                                           float* __restrict__ aT, const Geom s, int Mpad, float q, long g_off,
-                                                          float* __restrict__ gmax) {
+                                                          int second, float* __restrict__ gmax) {
     // tile: 32 rows (m) x 32 columns (gco); reads follow the source's contiguous axis, writes follow m
     __shared__ float ts[32][33], tg[32][33];
     __shared__ float wave_max[4];
@@ -102,24 +104,30 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(const float* __restric
     const int CO = s.COg * s.G;
     const int m0 = blockIdx.x * 32, c0 = blockIdx.y * 32;
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
-    auto factor = [&](long idx) -> float {
+    // -> the factor; `other` receives the value of the second array
+    auto factor = [&](long idx, float& other) -> float {
         const float g = gout[idx];
+        other = second == 1 ? g : 0.f;
         gmx = fmaxf(gmx, fabsf(g));
         if (q == 0.f) return g;
-        if (g_off != 0) return 1.0f / out[idx];
+        if (second == 1) return 1.0f / out[idx];
         if (g == 0.f) return 0.f;
         // the root in double precision (its relative error is multiplied by q in the terms); exp2(log2 / q) is
         // accurate to a few double ulps and several times cheaper than pow
         const double root = q == 1.f ? (double)fabsf(g) : exp2(log2((double)fabsf(g)) / (double)q);
-        return (float)(copysign(root, (double)g) / (double)out[idx]);
+        const double a = copysign(root, (double)g) / (double)out[idx];
+        const float af = (float)a;
+        if (second == 2) other = (float)(a - (double)af);
+        return af;
     };
     if (s.HW == 1) {
 #pragma unroll
         for (int r = ty; r < 32; r += 8) {
             const int m = m0 + r, c = c0 + tx;
             const bool ok = m < s.M && c < CO;
-            ts[r][tx] = ok ? factor((long)m * CO + c) : 0.f;
-            tg[r][tx] = ok && g_off != 0 ? gout[(long)m * CO + c] : 0.f;
+            float o = 0.f;
+            ts[r][tx] = ok ? factor((long)m * CO + c, o) : 0.f;
+            tg[r][tx] = o;
         }
     } else {
 #pragma unroll
@@ -128,8 +136,7 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(const float* __restric
             float v = 0.f, gv = 0.f;
             if (m < s.M && c < CO) {
                 const int b = m / s.HW, hw = m - b * s.HW;
-                v = factor(((long)b * CO + c) * s.HW + hw);
-                if (g_off != 0) gv = gout[((long)b * CO + c) * s.HW + hw];
+                v = factor(((long)b * CO + c) * s.HW + hw, gv);
             }
             ts[tx][cidx] = v;
             tg[tx][cidx] = gv;
@@ -151,7 +158,7 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(const float* __restric
         const int m = m0 + tx, c = c0 + cidx;
         if (m < Mpad && c < CO) {
             aT[(long)c * Mpad + m] = ts[tx][cidx];
-            if (g_off != 0) aT[g_off + (long)c * Mpad + m] = tg[tx][cidx];
+            if (second != 0) aT[g_off + (long)c * Mpad + m] = tg[tx][cidx];
         }
     }
 }
@@ -261,8 +268,10 @@ __global__ __launch_bounds__(kBoundProbeBlock) void bwd_bound_probe_kernel(const
 constexpr int kBwdTransposeMinHW = 16;
 
 // What the launcher decides from the shape and the exponent alone.
+constexpr float kBwdCompensateFromQ = 24.0f;
 struct BwdPlan {
     int ip;              // exponent variant of the kernels
+    bool second;         // the variant reads a second factor array
     int cfg;             // 0..2, 4: row-split workgroups of 16 / 8 / 4, 2 waves; 3: small-batch kernel
     int rows_per_wg;
     bool want_adaptive;  // large exponent on a problem worth the probes: skipping and plain variants are all queued
@@ -277,6 +286,10 @@ static BwdPlan plan_backward(const Geom& s, float p) {
     // Large exponents on problems worth the extra launches: the skipping variants (IP -3, -4) and the plain one
     // (IP -1) are all queued and device-side probes of the data open the gate of one of them.
     pl.want_adaptive = pl.ip == -1 && q >= 15.0f && ((double)s.M * s.COg * s.G * s.CIg >= 2e8 || skip_forced_on());
+    // large exponents: the product under the power is compensated (see bwd_terms), the pre-pass writes what every
+    // float32 factor dropped into a second array
+    if (pl.ip == -1 && q >= kBwdCompensateFromQ) pl.ip = -5;
+    pl.second = pl.ip == -2 || pl.ip == -5;
     pl.cfg = 3;
     if (!small) {
         // rows are padded to whole chunks of a workgroup's rows (512, 256 or 128): the configuration with the least
@@ -299,7 +312,7 @@ static BwdPlan plan_backward(const Geom& s, float p) {
 size_t norm_backward_scratch_bytes(const Geom& s, float p) {
     const BwdPlan pl = plan_backward(s, p);
     const size_t mpad = (size_t)ceil_div(s.M, pl.rows_per_wg) * pl.rows_per_wg;
-    return (size_t)s.COg * s.G * mpad * sizeof(float) * (pl.ip == -2 ? 2 : 1);
+    return (size_t)s.COg * s.G * mpad * sizeof(float) * (pl.second ? 2 : 1);
 }
 
 int launch_norm_backward(const float* gout, const float* x, const float* w, const float* out, const Geom& s, float* gx,
@@ -321,8 +334,8 @@ int launch_norm_backward(const float* gout, const float* x, const float* w, cons
 
     const size_t tbytes = (size_t)s.COg * s.G * P.Mpad * sizeof(float);
     float* aT = nullptr;
-    P.g_off = ip == -2 ? (long)s.COg * s.G * P.Mpad : 0;
-    NDIST_HIP_TRY(scratch_alloc((void**)&aT, ip == -2 ? 2 * tbytes : tbytes, st));
+    P.g_off = pl.second ? (long)s.COg * s.G * P.Mpad : 0;
+    NDIST_HIP_TRY(scratch_alloc((void**)&aT, pl.second ? 2 * tbytes : tbytes, st));
 
     int rc = 0;
     // (thin upper tail of |x - w|: skipping is up to twice as fast; many pairs near the maximum: it would be slower)
@@ -344,7 +357,7 @@ int launch_norm_backward(const float* gout, const float* x, const float* w, cons
     if (!rc) {
         dim3 grid(ceil_div(P.Mpad, 32), ceil_div(s.COg * s.G, 32));
         hipLaunchKernelGGL(bwd_prepare_kernel, grid, dim3(256), 0, st, out, gout, aT, s, P.Mpad, q, P.g_off,
-                           adaptive ? aux + 4 : (float*)nullptr);
+                           ip == -2 ? 1 : (ip == -5 ? 2 : 0), adaptive ? aux + 4 : (float*)nullptr);
         if (hip_failed(hipGetLastError())) rc = 4;
     }
     const long nx = (long)s.M * s.CIg * s.G;
@@ -445,9 +458,9 @@ int launch_norm_backward(const float* gout, const float* x, const float* w, cons
                     if (!rc) rc = launch_bwd_ip<-3>(a, P, cfg, grid, st);
                     P.gate2 = nullptr;
                     P.gate_sense = 0;
-                    if (!rc) rc = launch_bwd_ip<-1>(a, P, cfg, grid, st);
+                    if (!rc) rc = ip == -5 ? launch_bwd_ip<-5>(a, P, cfg, grid, st) : launch_bwd_ip<-1>(a, P, cfg, grid, st);
                 } else {
-                    rc = launch_bwd_ip<-1>(a, P, cfg, grid, st);
+                    rc = ip == -5 ? launch_bwd_ip<-5>(a, P, cfg, grid, st) : launch_bwd_ip<-1>(a, P, cfg, grid, st);
                 }
                 break;
         }

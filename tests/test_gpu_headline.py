@@ -140,6 +140,64 @@ def test_bound_forward(data, skip):
     assert_close(gw.cpu().numpy(), ew, what="grad_weight")
 
 
+def test_identity_initialised_layer_every_output():
+    """The shape the training and certification figures are quoted on: a 5120 x 5120 layer as the reference
+    initialises it (unit-variance weights with -10 planted on the diagonal, core/modules/norm_dist.py:18, 47-50),
+    batch 512, activations as a mean shift leaves them.  The library's default path there selects the hot k-tiles by
+    the rows of w.  Every output and code of the distance, of the interval bounds, of the joint calls and of the
+    calls with the weights' pre-pass kept is compared with the oracle (reference: core/cuda/inf_dist_cuda.cu:173-177,
+    bound_inf_dist_cuda.cu:203-213)."""
+    from core import _C
+    gen = torch.Generator().manual_seed(2021)
+    x = torch.randn(B, CI, 1, generator=gen) * 1.1
+    x -= x.mean(dim=0, keepdim=True)
+    w = torch.randn(CO, CI, generator=gen)
+    w[torch.arange(CO), torch.arange(CO) % CI] = -10.0
+    xl, xu = x - 8 / 255, x + 8 / 255
+    eo, ep = O.inf_dist_forward(x.numpy(), w.numpy())
+    el, eu, epl, epu = O.bound_inf_dist_forward(xl.numpy(), xu.numpy(), w.numpy())
+    xd, xld, xud, wd = x.cuda(), xl.cuda(), xu.cuda(), w.cuda()
+    new_f = lambda: torch.full((B, CO, 1), float("nan"), device="cuda")
+    new_i = lambda: torch.full((B, CO, 1), -7, device="cuda", dtype=torch.int32)
+    same = lambda t, e, what: np.testing.assert_array_equal(t.cpu().numpy(), e, err_msg=what)
+    out, pos = new_f(), new_i()
+    _C.inf_dist_forward(xd, wd, out, pos, 1)
+    same(out, eo, "distance"), same(pos, ep, "distance codes")
+    out = new_f()
+    _C.inf_dist_forward_nograd(xd, wd, out, 1)
+    same(out, eo, "distance, no codes")
+    yl, yu, pl, pu = new_f(), new_f(), new_i(), new_i()
+    _C.bound_inf_dist_forward(xld, xud, wd, yl, yu, pl, pu, 1)
+    same(yl, el, "lower"), same(yu, eu, "upper"), same(pl, epl, "lower codes"), same(pu, epu, "upper codes")
+    yl, yu = new_f(), new_f()
+    _C.bound_inf_dist_forward_nograd(xld, xud, wd, yl, yu, 1)
+    same(yl, el, "lower, no codes"), same(yu, eu, "upper, no codes")
+    out, pos, yl, yu, pl, pu = new_f(), new_i(), new_f(), new_f(), new_i(), new_i()
+    _C.inf_and_bound_forward(xd, xld, xud, wd, out, pos, yl, yu, pl, pu, 1)
+    same(out, eo, "joint distance"), same(pos, ep, "joint distance codes")
+    same(yl, el, "joint lower"), same(yu, eu, "joint upper")
+    same(pl, epl, "joint lower codes"), same(pu, epu, "joint upper codes")
+    out, yl, yu = new_f(), new_f(), new_f()
+    _C.inf_and_bound_forward_nograd(xd, xld, xud, wd, out, yl, yu, 1)
+    same(out, eo, "joint distance, no codes"), same(yl, el, "joint lower, no codes"), same(yu, eu, "joint upper, no codes")
+    cache = _C.weight_cache(wd, 1)
+    out = new_f()
+    _C.inf_dist_forward_nograd_cached(xd, wd, cache, out, 1)
+    same(out, eo, "distance, kept pre-pass")
+    out, yl, yu = new_f(), new_f(), new_f()
+    _C.inf_and_bound_forward_nograd_cached(xd, xld, xud, wd, cache, out, yl, yu, 1)
+    same(out, eo, "joint distance, kept pre-pass"), same(yl, el, "joint lower, kept pre-pass")
+    same(yu, eu, "joint upper, kept pre-pass")
+    # the hot-tile selection forced onto the rows of x (not chosen on this data: nearly every tile is hot there)
+    _C.set_hot_mode(2)
+    try:
+        out, pos = new_f(), new_i()
+        _C.inf_dist_forward(xd, wd, out, pos, 1)
+    finally:
+        _C.set_hot_mode(-1)
+    same(out, eo, "distance, x side forced"), same(pos, ep, "distance codes, x side forced")
+
+
 def test_config1_forward_p8_uniform_inputs():
     # forward only, p = 8: x uniform[0, 1) [512, 3072], w N(0, 1/3072) [5120, 3072]
     from core import _C
@@ -338,14 +396,14 @@ def test_config4_mlp_step_full_size():
         # The mean shift of the next layer makes every column of grad_output sum to zero, and the identity
         # initialisation gives every output one dominant term (|t| / out close to 1): grad_weight is then a sum of
         # terms that cancel to about 1e-5 of their size, and a float32 evaluation of the terms cannot be better than
-        # that amplification allows.  Tolerance: 1e-5, or eight times the error of the plain float32 yardstick (the
-        # factor test_gpu_modules.py uses for the same effect on the small stack).
+        # that amplification allows.  Tolerance: 1e-5, or twice the error of the plain float32 yardstick where that
+        # yardstick itself misses 1e-5.
         ex, _ = O.norm_dist_backward(gn[rows], xn[rows], wn, on[rows], 8.0, with_weight=False)
-        tol, _ = backward_tolerances(gn[rows], xn[rows], wn, on[rows], 8.0, 1, ex, None, factor=8.0)
+        tol, _ = backward_tolerances(gn[rows], xn[rows], wn, on[rows], 8.0, 1, ex, None)
         assert_close(gx.cpu().numpy()[rows], ex, tol=tol, what="layer %d grad_input rows" % li)
         cs = cols if ws.shape[0] > 64 else slice(0, ws.shape[0])
         _, ew = O.norm_dist_backward(gn[:, cs], xn, wn[cs], on[:, cs], 8.0)
-        _, tol = backward_tolerances(gn[:, cs], xn, wn[cs], on[:, cs], 8.0, 1, None, ew, factor=8.0)
+        _, tol = backward_tolerances(gn[:, cs], xn, wn[cs], on[:, cs], 8.0, 1, None, ew)
         print("layer %d: grad_weight tolerance %.2e" % (li, tol))
         assert_close(gw.cpu().numpy()[cs], ew, tol=tol, what="layer %d grad_weight slice" % li)
         lhs = float((gx.double() * xs.double()).sum() + (gw.double() * ws.double()).sum())

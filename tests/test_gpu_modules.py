@@ -141,7 +141,14 @@ def test_mlp_training_step_matches_float64_formulation(p):
             continue
         err = rel_err(a.grad.cpu().numpy(), b64.grad.numpy())
         yard = rel_err(b32.grad.cpu().numpy(), b64.grad.numpy())
-        assert err < max(5e-5, 8 * yard), (n, err, yard)
+        # a parameter's gradient has passed through up to four operator calls, each held to 1e-5 on its own; beyond
+        # that only where torch's own float32 evaluation of the stack misses the same bound, and then three times its
+        # error (the gradients of the mean-shifted layers cancel to ~1e-3 of their terms; the kernels' power carries
+        # one rounding more under the exponent than torch.pow, like the reference's, and the stack compounds it)
+        bound = 4 * TOL if yard <= 4 * TOL else 3 * yard
+        if bound > 4 * TOL:
+            print("relaxed %s: kernel %.3e, float32 yardstick %.3e, tolerance %.3e" % (n, err, yard, bound))
+        assert err < bound, (n, err, yard)
     for (n, a), (_, b) in zip(model.named_buffers(), ref64.named_buffers()):
         assert rel_err(a.cpu().numpy(), b.numpy()) < TOL, n
 

@@ -76,8 +76,9 @@ def test_forced_variants_at_extreme_scales(skip_mode, scale, mode):
     assert_close(out, O.norm_dist_forward(x, w, p), what="forward scale %g" % scale)
     ex, ew = O.norm_dist_backward(g, x, w, out, p)
     gx, gw = gpu_norm_backward(g, x, w, out, p)
-    assert_close(gx, ex, tol=2e-5, what="grad_input scale %g" % scale)
-    assert_close(gw, ew, tol=2e-5, what="grad_weight scale %g" % scale)
+    tol_x, tol_w = backward_tolerances(g, x, w, out, p, 1, ex, ew)  # 1e-5 unless plain float32 cannot reach it
+    assert_close(gx, ex, tol=tol_x, what="grad_input scale %g" % scale)
+    assert_close(gw, ew, tol=tol_w, what="grad_weight scale %g" % scale)
 
 
 def test_mode_is_reset():

@@ -1,13 +1,14 @@
 """The p = inf forwards with the pre-pass over the weights kept between calls (ndist_weight_cache_prepare and the
 *_nograd_cached entry points): bit-identical to the plain entry points, on problems that use the pre-pass (hot
-k-tiles, k-tile skipping) and on problems that ignore it; and the layer's use of it in evaluation: the cache follows
-the weights through in-place updates and moves."""
+k-tiles, k-tile skipping) and on problems that ignore it; and the layers' opt-in use of it (freeze_weights): nothing
+is kept unless asked, and what is kept is checked against the oracle through every kind of weight update."""
 import numpy as np
 import pytest
 import torch
 
 from core import _C
-from core.modules import NormDist
+from core.modules import NormDist, freeze_weights, unfreeze_weights
+from oracle import norm_dist_oracle as O
 
 pytestmark = pytest.mark.gpu
 
@@ -44,37 +45,93 @@ def test_cached_forwards_are_bit_identical(B, CO, CI, G, kind):
     assert torch.equal(r[0], ref)
 
 
-def test_layer_cache_follows_the_weights():
-    torch.manual_seed(1)
-    layer = NormDist(1024, 1024, bias=False, mean_shift=False).cuda().eval()
-    x = torch.randn(256, 1024, device="cuda")
+def _oracle_triple(layer, x, lo, up):
+    w = layer.weight.detach().cpu().numpy()
+    a = lambda t: t.detach().cpu().numpy()[:, :, None]
+    y = O.inf_dist_forward(a(x), w, with_pos=False)[0]
+    yl, yu, _, _ = O.bound_inf_dist_forward(a(lo), a(up), w, with_pos=False)
+    return [torch.from_numpy(t[:, :, 0]) for t in (y, yl, yu)]
 
-    def plain():
-        out = torch.empty(256, 1024, 1, device="cuda")
-        _C.inf_dist_forward_nograd(x.unsqueeze(-1).contiguous(), layer.weight.detach(), out, 1)
-        return out.squeeze(-1)
 
+def _certify(layer, x, lo, up):
     with torch.no_grad():
-        first = layer(x)[0]
-        assert torch.equal(first, plain())
-        buffer = layer._weight_cache._buffer
-        assert buffer is not None
-        assert torch.equal(layer(x)[0], first) and layer._weight_cache._buffer is buffer  # kept
-        layer.weight.add_(torch.randn_like(layer.weight))                                 # an optimizer-style update
-        assert torch.equal(layer(x)[0], plain()) and layer._weight_cache._buffer is not buffer
-        buffer = layer._weight_cache._buffer
-        layer.load_state_dict({"weight": torch.randn(1024, 1024)})
-        assert torch.equal(layer(x)[0], plain()) and layer._weight_cache._buffer is not buffer
-        lo, up = x - 0.1, x + 0.1
-        y, yl, yu = layer(x, lo, up)
-        r = [torch.empty(256, 1024, 1, device="cuda") for _ in range(3)]
-        _C.inf_and_bound_forward_nograd(*(t.unsqueeze(-1).contiguous() for t in (x, lo, up)), layer.weight.detach(), *r, 1)
-        assert all(torch.equal(a, b.squeeze(-1)) for a, b in zip((y, yl, yu), r))
+        return [t.cpu() for t in layer(x, lo, up)]
+
+
+def _same(got, want):
+    return all(torch.equal(a, b) for a, b in zip(got, want))
+
+
+def test_layers_keep_nothing_unless_asked():
+    """Evaluation without gradients keeps no state between calls by default (like the reference's layers): weights
+    rewritten through `.data`, which advances no version counter, are seen by the next certified evaluation."""
+    torch.manual_seed(1)
+    layer = NormDist(1024, 1024, bias=False, mean_shift=False, identity_val=10.0).cuda().eval()
+    x = torch.randn(256, 1024, device="cuda")
+    lo, up = x - 0.1, x + 0.1
+    assert _same(_certify(layer, x, lo, up), _oracle_triple(layer, x, lo, up))
+    assert layer._weight_cache._buffer is None
+    version = layer.weight._version
+    layer.weight.data.mul_(-0.5)                      # e.g. weight averaging, clipping, a hand-written update
+    layer.weight.data[:, :7] += 3.0
+    assert layer.weight._version == version           # invisible to torch
+    assert _same(_certify(layer, x, lo, up), _oracle_triple(layer, x, lo, up))
+    with torch.no_grad():
+        assert torch.equal(layer(x)[0].cpu(), _oracle_triple(layer, x, lo, up)[0])
+
+
+def test_frozen_weights_contract():
+    """freeze_weights(): the pre-pass is kept and reused; visible updates redo it; after a `.data` write the caller
+    freezes again; train(), load_state_dict() and device moves unfreeze."""
+    torch.manual_seed(2)
+    layer = NormDist(1024, 1024, bias=False, mean_shift=False, identity_val=10.0).cuda().eval()
+    x = torch.randn(256, 1024, device="cuda")
+    lo, up = x - 0.1, x + 0.1
+    cache = layer._weight_cache
+    assert layer.freeze_weights() and cache.frozen
+    buffer = cache._buffer
+    assert _same(_certify(layer, x, lo, up), _oracle_triple(layer, x, lo, up)) and cache._buffer is buffer
+    with torch.no_grad():
+        assert torch.equal(layer(x)[0].cpu(), _oracle_triple(layer, x, lo, up)[0]) and cache._buffer is buffer
+        layer.weight.add_(torch.randn_like(layer.weight))          # an optimizer-style update: version advances
+    assert _same(_certify(layer, x, lo, up), _oracle_triple(layer, x, lo, up)) and cache._buffer is not buffer
+    layer.weight.data.mul_(-0.5)                                   # invisible: the contract asks for a new freeze
+    layer.freeze_weights()
+    assert _same(_certify(layer, x, lo, up), _oracle_triple(layer, x, lo, up))
     layer.train()
-    before = layer._weight_cache._key
-    layer(x)          # training: the cache is left alone
-    assert layer._weight_cache._key == before
+    assert not cache.frozen and cache._buffer is None
+    layer.eval()
+    assert _same(_certify(layer, x, lo, up), _oracle_triple(layer, x, lo, up)) and cache._buffer is None
+    layer.freeze_weights()
+    layer.load_state_dict({"weight": torch.randn(1024, 1024)})
+    assert not cache.frozen
+    assert _same(_certify(layer, x, lo, up), _oracle_triple(layer, x, lo, up))
+    layer.freeze_weights()
+    layer.float()                                                  # any _apply (moves, casts) unfreezes
+    assert not cache.frozen
+    layer.freeze_weights()
+    with torch.enable_grad():                                      # with gradients the kept pre-pass is not used
+        layer(x)[0].sum().backward()
     assert "_weight_cache" not in layer.state_dict()
+    model = torch.nn.Sequential(layer, NormDist(1024, 64).cuda())
+    model.eval()
+    assert freeze_weights(model) == 2 and model[1]._weight_cache.frozen
+    unfreeze_weights(model)
+    assert not layer._weight_cache.frozen and not model[1]._weight_cache.frozen
+
+
+def test_non_contiguous_weights_are_never_cached():
+    torch.manual_seed(3)
+    layer = NormDist(640, 1280, bias=False, mean_shift=False).cuda().eval()
+    with torch.no_grad():
+        layer.weight = torch.nn.Parameter(torch.randn(640, 1280, device="cuda").t())   # [1280, 640], strided
+    assert not layer.weight.is_contiguous()
+    assert layer.freeze_weights() is False and not layer._weight_cache.frozen
+    x = torch.randn(200, 640, device="cuda")
+    lo, up = x - 0.1, x + 0.1
+    assert _same(_certify(layer, x, lo, up), _oracle_triple(layer, x, lo, up))
+    layer.weight.data.mul_(2.0)
+    assert _same(_certify(layer, x, lo, up), _oracle_triple(layer, x, lo, up))
 
 
 def test_cache_size_and_validation():

@@ -33,8 +33,19 @@ def l2_err(a, b):
     return float(np.linalg.norm(a - b) / (n if n > 0 else 1.0))
 
 
+class Tolerance(float):
+    """A tolerance beyond REL_TOL together with the error of the plain float32 evaluation that justified it."""
+    yardstick = None        # error of torch's float32 evaluation against the float64 oracle
+    reference_order = None  # error of the reference's order of operations in float32
+
+
 def assert_close(a, b, tol=REL_TOL, what=""):
     e, e2 = rel_err(a, b), l2_err(a, b)
+    if tol > REL_TOL:  # every comparison that needed more than the operator's bar says by how much, and why
+        known = isinstance(tol, Tolerance)
+        print("relaxed %s: kernel max-rel %.3e l2-rel %.3e; float32 torch %s, float32 in the reference's order %s; "
+              "tolerance %.3e" % (what, e, e2, "%.3e" % tol.yardstick if known else "n/a",
+                                  "%.3e" % tol.reference_order if known else "n/a", tol))
     assert e <= tol and e2 <= tol, "%s: max-rel %.3e, l2-rel %.3e (tol %.1e)" % (what, e, e2, tol)
 
 
@@ -64,16 +75,86 @@ def fp32_yardstick_backward(g, x, w, out, p, G=1):
     return gx.view(B, CI, HW).cpu().numpy(), gw.view(CO, CIg).cpu().numpy()
 
 
-def backward_tolerances(g, x, w, out, p, G, ex, ew, factor=8.0):
-    """Tolerances for (grad_x, grad_w) against the float64 oracle values ex, ew: the operator's 1e-5, or `factor`
-    times what the float32 yardstick itself reaches on the same inputs where that is larger (large p, or sums that
-    cancel).  The factor covers what the kernels' power carries beyond torch.pow: like the reference's
-    (core/cuda/norm_dist_cuda.cu:238-243, __powf) it is exp2(q * log2(u)) on the hardware transcendentals, whose
-    one-ulp errors and the rounding of the scaled difference are each multiplied by q = p - 1 as well."""
+def fp32_reference_order_backward(g, x, w, out, p, G=1):
+    """(grad_x, grad_w) evaluated in float32 in the ORDER OF OPERATIONS of the reference's kernels
+    (core/cuda/norm_dist_cuda.cu:238-243 with core/cuda/fast_pow.cuh:1-23): r = 1 / out rounded to float32,
+    u = (x - w) * r, the power by the reference's multiplication ladder for integral p - 1 <= 7 (its dispatch,
+    core/cuda/norm_dist.cpp:14-35) and as exp2(q * log2|u|) otherwise (what __powf computes, here with torch's float32
+    exp2 / log2, which are at least as accurate as the device intrinsics), times g, times the sign; sums by torch.sum
+    in float32.  Its error against the float64 oracle is what the reference's own arithmetic costs on these inputs."""
+    B, CI, HW = x.shape
+    CO = w.shape[0]
+    CIg, COg = CI // G, CO // G
+    xt = dev(x).view(B, G, 1, CIg, HW)
+    wt = dev(w).view(1, G, COg, CIg, 1)
+    rt = (1.0 / dev(out.astype(np.float32))).view(B, G, COg, 1, HW)
+    gt = dev(g).view(B, G, COg, 1, HW)
+    gx = torch.zeros(B, G, CIg, HW, dtype=torch.float32, device="cuda")
+    gw = torch.zeros(G, COg, CIg, dtype=torch.float32, device="cuda")
+    step = max(1, (1 << 25) // max(1, B * G * CIg * HW))
+    q = float(p) - 1.0
+    ip = int(q) if q == int(q) and 0 <= q <= 7 else -1
+    for c in range(0, COg, step):
+        t = xt - wt[:, :, c:c + step]
+        u = t * rt[:, :, c:c + step]
+        au = u.abs()
+        if ip == 0:
+            pw = torch.ones_like(u)
+        elif ip == 1:
+            pw = au
+        elif ip == 2:
+            pw = u * u
+        elif ip == 3:
+            pw = au * u * u
+        elif ip == 4:
+            t1 = u * u
+            pw = t1 * t1
+        elif ip == 5:
+            t1 = u * u
+            pw = au * t1 * t1
+        elif ip == 6:
+            t1 = u * u
+            pw = t1 * t1 * t1
+        elif ip == 7:
+            t1 = u * u
+            pw = au * t1 * t1 * t1
+        else:
+            pw = torch.exp2(torch.log2(au) * q)
+        term = gt[:, :, c:c + step] * pw * torch.where(t >= 0, 1.0, -1.0)
+        gx += term.sum(dim=2)
+        gw[:, c:c + step] -= term.sum(dim=(0, 4))
+    return gx.view(B, CI, HW).cpu().numpy(), gw.view(CO, CIg).cpu().numpy()
+
+
+def backward_tolerances(g, x, w, out, p, G, ex, ew, factor=2.0):
+    """Tolerances for (grad_x, grad_w) against the float64 oracle values ex, ew.  The operator's 1e-5 holds wherever
+    float32 can deliver it: the bound is raised only where a plain float32 evaluation of the same formula on the
+    same inputs misses 1e-5 ITSELF (sums that cancel; exponents in the hundreds, which multiply every rounding of
+    the scaled difference), and then to `factor` x the error of the worse of two such evaluations: torch's
+    (fp32_yardstick_backward: two roundings under a correctly rounded pow) and the reference's own order of
+    operations (fp32_reference_order_backward: three roundings under the power).  The factor covers what the
+    multiplication ladders of the kernels add to the latter on sums that cancel: grad_output is folded into the
+    per-(row, co) factor as a root, so the ladder's operands sit at arbitrary mantissa positions instead of just
+    below 1, where float32 rounds a factor sqrt(2) finer (measured: 1.5 x the reference's order on the mean-shifted
+    layers of the 6 x 5120 stack).  For large exponents (p - 1 >= 24) the kernels compensate the product under the
+    power and are far inside 1e-5 where both yardsticks miss it.  Every comparison that uses a raised bound prints
+    the kernel's error and both yardsticks beside it (assert_close)."""
     yx, yw = fp32_yardstick_backward(g, x, w, out, p, G)
-    ey = max(rel_err(yx, ex), l2_err(yx, ex)) if ex is not None else 0.0
-    ew_ = max(rel_err(yw, ew), l2_err(yw, ew)) if ew is not None else 0.0
-    return max(REL_TOL, factor * ey), max(REL_TOL, factor * ew_)
+    rx, rw = fp32_reference_order_backward(g, x, w, out, p, G)
+
+    def tolerance(y, r, e):
+        if e is None:
+            return REL_TOL
+        ey = max(rel_err(y, e), l2_err(y, e))
+        er = max(rel_err(r, e), l2_err(r, e))
+        worst = max(ey, er)
+        if worst <= REL_TOL:
+            return REL_TOL
+        t = Tolerance(factor * worst)
+        t.yardstick, t.reference_order = ey, er
+        return t
+
+    return tolerance(yx, rx, ex), tolerance(yw, rw, ew)
 
 
 # ---- entry-point wrappers (outputs allocated by the caller, as the operator's contract requires) -----------
