@@ -64,8 +64,9 @@ int ndist_last_kernel_ms(float* ms);
  * several variants of its kernels and lets device-side probes of the data choose one.  skip: -1 the probes decide
  * (default), 0 never, 1 always run the pair-skipping variants (forced on, also for small problems); bounds: the same
  * for the choice between the two skipping variants of the backward.  skip also governs the k-tile skipping of
- * the p = inf and interval-bound forwards (on by default for large fully-connected problems).  Process-wide.  Initial values can be given in
- * the environment: NORM_DIST_SKIP, NORM_DIST_BWD_BOUNDS = 0 / 1.  Results agree within the operator's tolerance
+ * the p = inf and interval-bound forwards (on by default for large fully-connected problems).  The setting belongs to the
+ * calling host thread (it governs the entry points that thread calls afterwards; other threads are unaffected); -1
+ * returns to the value the environment gave when the library was loaded: NORM_DIST_SKIP, NORM_DIST_BWD_BOUNDS = 0 / 1.  Results agree within the operator's tolerance
  * whichever variant runs. */
 void ndist_set_skip_mode(int skip, int bounds);
 /* Tuning and test aid, no counterpart in the reference.  On the problems whose p = inf forward skips k-tiles the
@@ -73,15 +74,18 @@ void ndist_set_skip_mode(int skip, int bounds);
  * maximum (activations with a few outliers against small weights; weights with one large planted entry per row) and
  * then computes the outputs from those tiles alone; results are bit-identical either way.  mode: -1 the counts
  * decide (default), 0 never, 1 always the cheaper side, 2 always the rows of x, 3 always the rows of w.
- * Process-wide; initial value from NORM_DIST_HOT. */
+ * Per calling host thread, like ndist_set_skip_mode; -1 returns to the value of NORM_DIST_HOT at load time (or to
+ * the default). */
 void ndist_set_hot_mode(int mode);
 /* Tuning and test aid, no counterpart in the reference.  For 10 < p <= 48 in the fully connected layout the forward
  * normalises the sum by a bound of the maximum known before the reduction starts (largest |x| of the row plus
  * largest |w|) and so needs one pass over the pairs instead of two; outputs whose sum leaves the safe float range
  * under that bound are recomputed with their exact maximum.  mode: -1 for problems of 2e7 pairs and more (default),
- * 0 never, 1 whenever the layout allows.  Process-wide; initial value from NORM_DIST_ROW_SCALE.  Results agree within
+ * 0 never, 1 whenever the layout allows.  Per calling host thread; -1 returns to NORM_DIST_ROW_SCALE (or the default).  Results agree within
  * the operator's tolerance either way. */
 void ndist_set_scaled_mode(int mode);
+/* The calling host thread's current values of the three settings above (null pointers are skipped). */
+void ndist_get_modes(int* skip, int* bounds, int* hot, int* scaled);
 /* No counterpart in the reference (PyTorch's caching allocator plays this role there).  Entry points that need
  * temporary device memory (finite-p backward, forwards whose k range is split over workgroups, the large-p paths,
  * the conv fallback) take it from arenas the library keeps per (device, stream): allocated with hipMalloc the first
@@ -130,7 +134,12 @@ int ndist_norm_dist_backward_input_weight(const float* grad_output, const float*
  * return NDIST_ERR_TOO_LARGE before anything is launched (B*HW x CO up to 6.29 M, e.g. 512 x 5120 twice over); the
  * conv layout runs without the transposed copies of the allocating entry point when they do not fit.  All calls on
  * one GPU share that GPU's array: calls that overlap in time on one device (two streams, two threads) race; calls
- * queued on one stream do not.  Results are those of ndist_norm_dist_backward_input_weight. */
+ * queued on one stream do not.  Results are those of ndist_norm_dist_backward_input_weight.
+ * Under graph capture: the array's device address and the device's properties are looked up once per device, by
+ * ndist_noalloc_prepare() or by the first call made outside a capture; a call on a capturing stream that finds
+ * them missing returns NDIST_ERR_CAPTURE and launches nothing.  A graph that holds such a call also holds the
+ * array's address: replays race with any other use of the array on that GPU that overlaps them in time. */
+int ndist_noalloc_prepare(void); /* once per device, that device current, outside any capture; no counterpart either */
 int ndist_norm_dist_backward_input_weight_noalloc(const float* grad_output, const float* input, const float* weight,
                                                   const float* output, int B, int CO, int CI, int G, int HW,
                                                   float* grad_input, float* grad_weight, float p,

@@ -67,6 +67,8 @@ _lib.ndist_set_hot_mode.argtypes = [ctypes.c_int]
 _lib.ndist_set_hot_mode.restype = None
 _lib.ndist_set_scaled_mode.argtypes = [ctypes.c_int]
 _lib.ndist_set_scaled_mode.restype = None
+_lib.ndist_get_modes.argtypes = [ctypes.POINTER(ctypes.c_int)] * 4
+_lib.ndist_get_modes.restype = None
 _lib.ndist_release_scratch.argtypes = []
 _lib.ndist_release_scratch.restype = ctypes.c_int
 _lib.ndist_last_kernel_ms.argtypes = [ctypes.POINTER(ctypes.c_float)]
@@ -75,6 +77,8 @@ _lib.ndist_scratch_counters.argtypes = [ctypes.POINTER(ctypes.c_long), ctypes.PO
 _lib.ndist_scratch_counters.restype = None
 _lib.ndist_noalloc_scratch_bytes.argtypes = []
 _lib.ndist_noalloc_scratch_bytes.restype = ctypes.c_size_t
+_lib.ndist_noalloc_prepare.argtypes = []
+_lib.ndist_noalloc_prepare.restype = ctypes.c_int
 
 _DIMS = (_I, _I, _I, _I, _I)
 _norm_fwd = _sig("ndist_norm_dist_forward", _P, _P, *_DIMS, _P, _F, _P)
@@ -154,7 +158,9 @@ def set_profiling(enable):
 
 def set_skip_mode(skip=-1, bounds=-1):
     """Tuning / test aid: -1 lets the device-side probes choose the large-p kernel variants (default), 0 / 1 forces
-    the pair-skipping variants off / on; `bounds` likewise for the two skipping variants of the backward."""
+    the pair-skipping variants off / on; `bounds` likewise for the two skipping variants of the backward.  Like the
+    two settings below it belongs to the calling host thread: the entry points this thread calls afterwards follow
+    it, other threads (autograd's backward threads among them) do not."""
     _lib.ndist_set_skip_mode(int(skip), int(bounds))
 
 
@@ -168,6 +174,13 @@ def set_scaled_mode(mode=-1):
     """Tuning / test aid for the one-pass normalised forward (10 < p <= 48, fully connected layout): -1 from 2e7
     pairs on (default), 0 never, 1 whenever the layout allows."""
     _lib.ndist_set_scaled_mode(int(mode))
+
+
+def get_modes():
+    """(skip, bounds, hot, scaled) as the calling thread has them (see set_skip_mode, set_hot_mode, set_scaled_mode)."""
+    v = [ctypes.c_int(-9) for _ in range(4)]
+    _lib.ndist_get_modes(*(ctypes.byref(c) for c in v))
+    return tuple(c.value for c in v)
 
 
 def release_scratch():
@@ -201,6 +214,26 @@ def _check(dtype, **tensors):
         elif t.device != dev:
             raise RuntimeError("%s is on %s, expected %s" % (name, t.device, dev))
     return dev
+
+
+def _agree(B, CO, CI, G, HW, **tensors):
+    """Shape agreement of one operator call, by argument name: input-like tensors are [B, CI, HW], output-like ones
+    (outputs, their gradients, arg-max codes) [B, CO, HW], weights [CO, CI / G].  The kernels index every tensor from
+    these five numbers alone, so a tensor of another size would be read or written out of bounds."""
+    if G <= 0 or CI % G or CO % G:
+        raise RuntimeError("groups (%d) must divide the %d input and the %d output features" % (G, CI, CO))
+    for name, t in tensors.items():
+        if name == "cache":
+            continue
+        base = name[5:] if name.startswith("grad_") else name
+        if base.startswith("input"):
+            want = (B, CI, HW)
+        elif base.startswith("weight"):
+            want = (CO, CI // G)
+        else:
+            want = (B, CO, HW)
+        if tuple(t.shape) != want:
+            raise RuntimeError("%s must be %s, got %s" % (name, list(want), list(t.shape)))
 
 
 def _run(fn, dev, *args, stream=None):
@@ -243,6 +276,7 @@ def norm_dist_forward(input, weight, output, G, p):
         return _ext_call(_ext.norm_dist_forward, input, weight, output, G, p)
     dev = _check({}, input=input, weight=weight, output=output)
     B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
+    _agree(B, CO, CI, G, HW, input=input, weight=weight, output=output)
     _run(_norm_fwd, dev, _p(input), _p(weight), B, CO, CI, G, HW, _p(output), p)
 
 
@@ -251,6 +285,7 @@ def norm_dist_forward_with_max(input, weight, max_output, output, G, p):
         return _ext_call(_ext.norm_dist_forward_with_max, input, weight, max_output, output, G, p)
     dev = _check({}, input=input, weight=weight, max_output=max_output, output=output)
     B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
+    _agree(B, CO, CI, G, HW, input=input, weight=weight, max_output=max_output, output=output)
     _run(_norm_fwd_max, dev, _p(input), _p(weight), _p(max_output), B, CO, CI, G, HW, _p(output), p)
 
 
@@ -259,6 +294,7 @@ def norm_dist_backward_input(grad_output, input, weight, output, grad_input, G, 
         return _ext_call(_ext.norm_dist_backward_input, grad_output, input, weight, output, grad_input, G, p)
     dev = _check({}, grad_output=grad_output, input=input, weight=weight, output=output, grad_input=grad_input)
     B, CO, CI, HW = grad_output.size(0), output.size(1), input.size(1), input.size(2)
+    _agree(B, CO, CI, G, HW, grad_output=grad_output, input=input, weight=weight, output=output, grad_input=grad_input)
     _run(_norm_bwd_x, dev, _p(grad_output), _p(input), _p(weight), _p(output), B, CO, CI, G, HW, _p(grad_input), p)
 
 
@@ -268,6 +304,7 @@ def norm_dist_backward_input_weight(grad_output, input, weight, output, grad_inp
     dev = _check({}, grad_output=grad_output, input=input, weight=weight, output=output, grad_input=grad_input,
                  grad_weight=grad_weight)
     B, CO, CI, HW = grad_output.size(0), output.size(1), input.size(1), input.size(2)
+    _agree(B, CO, CI, G, HW, grad_output=grad_output, input=input, weight=weight, output=output, grad_input=grad_input, grad_weight=grad_weight)
     _run(_norm_bwd_xw, dev, _p(grad_output), _p(input), _p(weight), _p(output), B, CO, CI, G, HW,
          _p(grad_input), _p(grad_weight), p)
 
@@ -282,6 +319,7 @@ def norm_dist_backward_input_weight_noalloc(grad_output, input, weight, output, 
     dev = _check({}, grad_output=grad_output, input=input, weight=weight, output=output, grad_input=grad_input,
                  grad_weight=grad_weight)
     B, CO, CI, HW = grad_output.size(0), output.size(1), input.size(1), input.size(2)
+    _agree(B, CO, CI, G, HW, grad_output=grad_output, input=input, weight=weight, output=output, grad_input=grad_input, grad_weight=grad_weight)
     _run(_norm_bwd_xw_noalloc, dev, _p(grad_output), _p(input), _p(weight), _p(output), B, CO, CI, G, HW,
          _p(grad_input), _p(grad_weight), p, stream=stream)
 
@@ -291,6 +329,7 @@ def inf_dist_forward(input, weight, output, pos, G):
         return _ext_call(_ext.inf_dist_forward, input, weight, output, pos, G)
     dev = _check(_INT, input=input, weight=weight, output=output, pos=pos)
     B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
+    _agree(B, CO, CI, G, HW, input=input, weight=weight, output=output, pos=pos)
     _run(_inf_fwd, dev, _p(input), _p(weight), B, CO, CI, G, HW, _p(output), _p(pos))
 
 
@@ -299,6 +338,7 @@ def inf_dist_forward_nograd(input, weight, output, G):
         return _ext_call(_ext.inf_dist_forward_nograd, input, weight, output, G)
     dev = _check({}, input=input, weight=weight, output=output)
     B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
+    _agree(B, CO, CI, G, HW, input=input, weight=weight, output=output)
     _run(_inf_fwd_ng, dev, _p(input), _p(weight), B, CO, CI, G, HW, _p(output))
 
 
@@ -307,6 +347,7 @@ def inf_dist_backward_input(grad_output, pos, grad_input, G):
         return _ext_call(_ext.inf_dist_backward_input, grad_output, pos, grad_input, G)
     dev = _check(_INT, grad_output=grad_output, pos=pos, grad_input=grad_input)
     B, CO, CI, HW = grad_output.size(0), grad_output.size(1), grad_input.size(1), grad_input.size(2)
+    _agree(B, CO, CI, G, HW, grad_output=grad_output, pos=pos, grad_input=grad_input)
     _run(_inf_bwd_x, dev, _p(grad_output), _p(pos), B, CO, CI, G, HW, _p(grad_input))
 
 
@@ -315,6 +356,7 @@ def inf_dist_backward_input_weight(grad_output, pos, grad_input, grad_weight, G)
         return _ext_call(_ext.inf_dist_backward_input_weight, grad_output, pos, grad_input, grad_weight, G)
     dev = _check(_INT, grad_output=grad_output, pos=pos, grad_input=grad_input, grad_weight=grad_weight)
     B, CO, CI, HW = grad_output.size(0), grad_output.size(1), grad_weight.size(1) * G, grad_output.size(2)
+    _agree(B, CO, CI, G, HW, grad_output=grad_output, pos=pos, grad_input=grad_input, grad_weight=grad_weight)
     _run(_inf_bwd_xw, dev, _p(grad_output), _p(pos), B, CO, CI, G, HW, _p(grad_input), _p(grad_weight))
 
 
@@ -323,6 +365,7 @@ def bound_inf_dist_forward_nograd(inputL, inputU, weight, outputL, outputU, G):
         return _ext_call(_ext.bound_inf_dist_forward_nograd, inputL, inputU, weight, outputL, outputU, G)
     dev = _check({}, inputL=inputL, inputU=inputU, weight=weight, outputL=outputL, outputU=outputU)
     B, CO, CI, HW = inputL.size(0), outputL.size(1), inputL.size(1), inputL.size(2)
+    _agree(B, CO, CI, G, HW, inputL=inputL, inputU=inputU, weight=weight, outputL=outputL, outputU=outputU)
     _run(_bnd_fwd_ng, dev, _p(inputL), _p(inputU), _p(weight), B, CO, CI, G, HW, _p(outputL), _p(outputU))
 
 
@@ -332,6 +375,7 @@ def bound_inf_dist_forward(inputL, inputU, weight, outputL, outputU, posL, posU,
     dev = _check(_INT, inputL=inputL, inputU=inputU, weight=weight, outputL=outputL, outputU=outputU,
                  posL=posL, posU=posU)
     B, CO, CI, HW = inputL.size(0), outputL.size(1), inputL.size(1), inputL.size(2)
+    _agree(B, CO, CI, G, HW, inputL=inputL, inputU=inputU, weight=weight, outputL=outputL, outputU=outputU, posL=posL, posU=posU)
     _run(_bnd_fwd, dev, _p(inputL), _p(inputU), _p(weight), B, CO, CI, G, HW, _p(outputL), _p(outputU),
          _p(posL), _p(posU))
 
@@ -342,6 +386,7 @@ def bound_inf_dist_backward_input(grad_outputL, grad_outputU, posL, posU, grad_i
     dev = _check(_INT, grad_outputL=grad_outputL, grad_outputU=grad_outputU, posL=posL, posU=posU,
                  grad_inputL=grad_inputL, grad_inputU=grad_inputU)
     B, CO, CI, HW = grad_outputL.size(0), grad_outputL.size(1), grad_inputL.size(1), grad_inputL.size(2)
+    _agree(B, CO, CI, G, HW, grad_outputL=grad_outputL, grad_outputU=grad_outputU, posL=posL, posU=posU, grad_inputL=grad_inputL, grad_inputU=grad_inputU)
     _run(_bnd_bwd_x, dev, _p(grad_outputL), _p(grad_outputU), _p(posL), _p(posU), B, CO, CI, G, HW,
          _p(grad_inputL), _p(grad_inputU))
 
@@ -353,6 +398,7 @@ def bound_inf_dist_backward_input_weight(grad_outputL, grad_outputU, posL, posU,
     dev = _check(_INT, grad_outputL=grad_outputL, grad_outputU=grad_outputU, posL=posL, posU=posU,
                  grad_inputL=grad_inputL, grad_inputU=grad_inputU, grad_weight=grad_weight)
     B, CO, CI, HW = grad_outputL.size(0), grad_outputL.size(1), grad_weight.size(1) * G, grad_outputL.size(2)
+    _agree(B, CO, CI, G, HW, grad_outputL=grad_outputL, grad_outputU=grad_outputU, posL=posL, posU=posU, grad_inputL=grad_inputL, grad_inputU=grad_inputU, grad_weight=grad_weight)
     _run(_bnd_bwd_xw, dev, _p(grad_outputL), _p(grad_outputU), _p(posL), _p(posU), B, CO, CI, G, HW,
          _p(grad_inputL), _p(grad_inputU), _p(grad_weight))
 
@@ -366,6 +412,7 @@ def inf_and_bound_forward_nograd(input, inputL, inputU, weight, output, outputL,
     dev = _check({}, input=input, inputL=inputL, inputU=inputU, weight=weight, output=output, outputL=outputL,
                  outputU=outputU)
     B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
+    _agree(B, CO, CI, G, HW, input=input, inputL=inputL, inputU=inputU, weight=weight, output=output, outputL=outputL, outputU=outputU)
     _run(_joint_ng, dev, _p(input), _p(inputL), _p(inputU), _p(weight), B, CO, CI, G, HW, _p(output), _p(outputL),
          _p(outputU))
 
@@ -387,6 +434,7 @@ def weight_cache(weight, G):
 def inf_dist_forward_nograd_cached(input, weight, cache, output, G):
     dev = _check({}, input=input, weight=weight, cache=cache, output=output)
     B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
+    _agree(B, CO, CI, G, HW, input=input, weight=weight, cache=cache, output=output)
     _run(_inf_ng_cached, dev, _p(input), _p(weight), _p(cache), B, CO, CI, G, HW, _p(output))
 
 
@@ -394,6 +442,7 @@ def inf_and_bound_forward_nograd_cached(input, inputL, inputU, weight, cache, ou
     dev = _check({}, input=input, inputL=inputL, inputU=inputU, weight=weight, cache=cache, output=output,
                  outputL=outputL, outputU=outputU)
     B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
+    _agree(B, CO, CI, G, HW, input=input, inputL=inputL, inputU=inputU, weight=weight, cache=cache, output=output, outputL=outputL, outputU=outputU)
     _run(_joint_ng_cached, dev, _p(input), _p(inputL), _p(inputU), _p(weight), _p(cache), B, CO, CI, G, HW, _p(output),
          _p(outputL), _p(outputU))
 
@@ -406,6 +455,7 @@ def inf_and_bound_forward(input, inputL, inputU, weight, output, pos, outputL, o
     dev = _check(_INT, input=input, inputL=inputL, inputU=inputU, weight=weight, output=output, pos=pos,
                  outputL=outputL, outputU=outputU, posL=posL, posU=posU)
     B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
+    _agree(B, CO, CI, G, HW, input=input, inputL=inputL, inputU=inputU, weight=weight, output=output, pos=pos, outputL=outputL, outputU=outputU, posL=posL, posU=posU)
     _run(_joint, dev, _p(input), _p(inputL), _p(inputU), _p(weight), B, CO, CI, G, HW, _p(output), _p(pos), _p(outputL),
          _p(outputU), _p(posL), _p(posU))
 

@@ -61,10 +61,30 @@ int32_t* IM(Tensor& t) { return t.data_ptr<int32_t>(); }
 
 void need3d(const Tensor& t, const char* name) { TORCH_CHECK(t.dim() == 3, name, " must be [B, C, HW]"); }
 
+// Shape agreement of one operator call (the kernels index every tensor from B, CO, CI, G, HW alone: a tensor of
+// another size would be read or written out of bounds).  ins are [B, CI, HW], outs [B, CO, HW], ws [CO, CI / G].
+using Named = std::pair<const char*, const Tensor*>;
+void agree(int64_t B, int64_t CO, int64_t CI, int64_t G, int64_t HW, std::initializer_list<Named> ins,
+           std::initializer_list<Named> outs, std::initializer_list<Named> ws) {
+    TORCH_CHECK(G > 0 && CI % G == 0 && CO % G == 0, "groups (", G, ") must divide the ", CI, " input and the ", CO,
+                " output features");
+    for (const Named& n : ins)
+        TORCH_CHECK(n.second->dim() == 3 && n.second->size(0) == B && n.second->size(1) == CI && n.second->size(2) == HW,
+                    n.first, " must be [", B, ", ", CI, ", ", HW, "], got ", n.second->sizes());
+    for (const Named& n : outs)
+        TORCH_CHECK(n.second->dim() == 3 && n.second->size(0) == B && n.second->size(1) == CO && n.second->size(2) == HW,
+                    n.first, " must be [", B, ", ", CO, ", ", HW, "], got ", n.second->sizes());
+    for (const Named& n : ws)
+        TORCH_CHECK(n.second->dim() == 2 && n.second->size(0) == CO && n.second->size(1) * G == CI, n.first, " must be [",
+                    CO, ", ", CI / G, "], got ", n.second->sizes());
+}
+#define NM(t) Named{#t, &t}
+
 // ---- finite p --------------------------------------------------------------------------------------------------
 void norm_dist_forward(const Tensor& input, const Tensor& weight, Tensor& output, int G, float p) {
     const int dev = check_all({{"input", input, false}, {"weight", weight, false}, {"output", output, false}});
     need3d(input, "input"); need3d(output, "output");
+    agree(input.size(0), output.size(1), input.size(1), G, input.size(2), {NM(input)}, {NM(output)}, {NM(weight)});
     Launch L(dev);
     raise_on(ndist_norm_dist_forward(F(input), F(weight), input.size(0), output.size(1), input.size(1), G, input.size(2),
                                      FM(output), p, L.stream), "norm_dist_forward");
@@ -75,6 +95,7 @@ void norm_dist_forward_with_max(const Tensor& input, const Tensor& weight, const
     const int dev = check_all({{"input", input, false}, {"weight", weight, false}, {"max_output", max_output, false},
                                {"output", output, false}});
     need3d(input, "input"); need3d(output, "output");
+    agree(input.size(0), output.size(1), input.size(1), G, input.size(2), {NM(input)}, {NM(output), NM(max_output)}, {NM(weight)});
     Launch L(dev);
     raise_on(ndist_norm_dist_forward_with_max(F(input), F(weight), F(max_output), input.size(0), output.size(1),
                                               input.size(1), G, input.size(2), FM(output), p, L.stream),
@@ -86,6 +107,7 @@ void norm_dist_backward_input(const Tensor& grad_output, const Tensor& input, co
     const int dev = check_all({{"grad_output", grad_output, false}, {"input", input, false}, {"weight", weight, false},
                                {"output", output, false}, {"grad_input", grad_input, false}});
     need3d(input, "input"); need3d(output, "output");
+    agree(input.size(0), output.size(1), input.size(1), G, input.size(2), {NM(input), NM(grad_input)}, {NM(output), NM(grad_output)}, {NM(weight)});
     Launch L(dev);
     raise_on(ndist_norm_dist_backward_input(F(grad_output), F(input), F(weight), F(output), grad_output.size(0),
                                             output.size(1), input.size(1), G, input.size(2), FM(grad_input), p, L.stream),
@@ -98,6 +120,7 @@ void norm_dist_backward_input_weight(const Tensor& grad_output, const Tensor& in
                                {"output", output, false}, {"grad_input", grad_input, false},
                                {"grad_weight", grad_weight, false}});
     need3d(input, "input"); need3d(output, "output");
+    agree(input.size(0), output.size(1), input.size(1), G, input.size(2), {NM(input), NM(grad_input)}, {NM(output), NM(grad_output)}, {NM(weight), NM(grad_weight)});
     Launch L(dev);
     raise_on(ndist_norm_dist_backward_input_weight(F(grad_output), F(input), F(weight), F(output), grad_output.size(0),
                                                    output.size(1), input.size(1), G, input.size(2), FM(grad_input),
@@ -113,6 +136,7 @@ void norm_dist_backward_input_weight_noalloc(const Tensor& grad_output, const Te
                                {"output", output, false}, {"grad_input", grad_input, false},
                                {"grad_weight", grad_weight, false}});
     need3d(input, "input"); need3d(output, "output");
+    agree(input.size(0), output.size(1), input.size(1), G, input.size(2), {NM(input), NM(grad_input)}, {NM(output), NM(grad_output)}, {NM(weight), NM(grad_weight)});
     Launch L(dev);
     raise_on(ndist_norm_dist_backward_input_weight_noalloc(F(grad_output), F(input), F(weight), F(output),
                                                            grad_output.size(0), output.size(1), input.size(1), G,
@@ -125,6 +149,7 @@ void inf_dist_forward(const Tensor& input, const Tensor& weight, Tensor& output,
     const int dev = check_all({{"input", input, false}, {"weight", weight, false}, {"output", output, false},
                                {"pos", pos, true}});
     need3d(input, "input"); need3d(output, "output");
+    agree(input.size(0), output.size(1), input.size(1), G, input.size(2), {NM(input)}, {NM(output), NM(pos)}, {NM(weight)});
     Launch L(dev);
     raise_on(ndist_inf_dist_forward(F(input), F(weight), input.size(0), output.size(1), input.size(1), G, input.size(2),
                                     FM(output), IM(pos), L.stream), "inf_dist_forward");
@@ -133,6 +158,7 @@ void inf_dist_forward(const Tensor& input, const Tensor& weight, Tensor& output,
 void inf_dist_forward_nograd(const Tensor& input, const Tensor& weight, Tensor& output, int G) {
     const int dev = check_all({{"input", input, false}, {"weight", weight, false}, {"output", output, false}});
     need3d(input, "input"); need3d(output, "output");
+    agree(input.size(0), output.size(1), input.size(1), G, input.size(2), {NM(input)}, {NM(output)}, {NM(weight)});
     Launch L(dev);
     raise_on(ndist_inf_dist_forward_nograd(F(input), F(weight), input.size(0), output.size(1), input.size(1), G,
                                            input.size(2), FM(output), L.stream), "inf_dist_forward_nograd");
@@ -141,6 +167,7 @@ void inf_dist_forward_nograd(const Tensor& input, const Tensor& weight, Tensor& 
 void inf_dist_backward_input(const Tensor& grad_output, const Tensor& pos, Tensor& grad_input, int G) {
     const int dev = check_all({{"grad_output", grad_output, false}, {"pos", pos, true}, {"grad_input", grad_input, false}});
     need3d(grad_output, "grad_output"); need3d(grad_input, "grad_input");
+    agree(grad_output.size(0), grad_output.size(1), grad_input.size(1), G, grad_output.size(2), {NM(grad_input)}, {NM(grad_output), NM(pos)}, {});
     Launch L(dev);
     raise_on(ndist_inf_dist_backward_input(F(grad_output), I(pos), grad_output.size(0), grad_output.size(1),
                                            grad_input.size(1), G, grad_input.size(2), FM(grad_input), L.stream),
@@ -152,6 +179,8 @@ void inf_dist_backward_input_weight(const Tensor& grad_output, const Tensor& pos
     const int dev = check_all({{"grad_output", grad_output, false}, {"pos", pos, true}, {"grad_input", grad_input, false},
                                {"grad_weight", grad_weight, false}});
     need3d(grad_output, "grad_output");
+    TORCH_CHECK(grad_weight.dim() == 2, "grad_weight must be [CO, CI / G]");
+    agree(grad_output.size(0), grad_output.size(1), grad_weight.size(1) * G, G, grad_output.size(2), {NM(grad_input)}, {NM(grad_output), NM(pos)}, {NM(grad_weight)});
     Launch L(dev);
     raise_on(ndist_inf_dist_backward_input_weight(F(grad_output), I(pos), grad_output.size(0), grad_output.size(1),
                                                   grad_weight.size(1) * G, G, grad_output.size(2), FM(grad_input),
@@ -166,6 +195,7 @@ void bound_inf_dist_forward(const Tensor& inputL, const Tensor& inputU, const Te
                                {"outputL", outputL, false}, {"outputU", outputU, false}, {"posL", posL, true},
                                {"posU", posU, true}});
     need3d(inputL, "inputL"); need3d(outputL, "outputL");
+    agree(inputL.size(0), outputL.size(1), inputL.size(1), G, inputL.size(2), {NM(inputL), NM(inputU)}, {NM(outputL), NM(outputU), NM(posL), NM(posU)}, {NM(weight)});
     Launch L(dev);
     raise_on(ndist_bound_inf_dist_forward(F(inputL), F(inputU), F(weight), inputL.size(0), outputL.size(1), inputL.size(1),
                                           G, inputL.size(2), FM(outputL), FM(outputU), IM(posL), IM(posU), L.stream),
@@ -177,6 +207,7 @@ void bound_inf_dist_forward_nograd(const Tensor& inputL, const Tensor& inputU, c
     const int dev = check_all({{"inputL", inputL, false}, {"inputU", inputU, false}, {"weight", weight, false},
                                {"outputL", outputL, false}, {"outputU", outputU, false}});
     need3d(inputL, "inputL"); need3d(outputL, "outputL");
+    agree(inputL.size(0), outputL.size(1), inputL.size(1), G, inputL.size(2), {NM(inputL), NM(inputU)}, {NM(outputL), NM(outputU)}, {NM(weight)});
     Launch L(dev);
     raise_on(ndist_bound_inf_dist_forward_nograd(F(inputL), F(inputU), F(weight), inputL.size(0), outputL.size(1),
                                                  inputL.size(1), G, inputL.size(2), FM(outputL), FM(outputU), L.stream),
@@ -189,6 +220,7 @@ void bound_inf_dist_backward_input(const Tensor& grad_outputL, const Tensor& gra
                                {"posL", posL, true}, {"posU", posU, true}, {"grad_inputL", grad_inputL, false},
                                {"grad_inputU", grad_inputU, false}});
     need3d(grad_outputL, "grad_outputL"); need3d(grad_inputL, "grad_inputL");
+    agree(grad_outputL.size(0), grad_outputL.size(1), grad_inputL.size(1), G, grad_outputL.size(2), {NM(grad_inputL), NM(grad_inputU)}, {NM(grad_outputL), NM(grad_outputU), NM(posL), NM(posU)}, {});
     Launch L(dev);
     raise_on(ndist_bound_inf_dist_backward_input(F(grad_outputL), F(grad_outputU), I(posL), I(posU), grad_outputL.size(0),
                                                  grad_outputL.size(1), grad_inputL.size(1), G, grad_inputL.size(2),
@@ -203,6 +235,8 @@ void bound_inf_dist_backward_input_weight(const Tensor& grad_outputL, const Tens
                                {"posL", posL, true}, {"posU", posU, true}, {"grad_inputL", grad_inputL, false},
                                {"grad_inputU", grad_inputU, false}, {"grad_weight", grad_weight, false}});
     need3d(grad_outputL, "grad_outputL");
+    TORCH_CHECK(grad_weight.dim() == 2, "grad_weight must be [CO, CI / G]");
+    agree(grad_outputL.size(0), grad_outputL.size(1), grad_weight.size(1) * G, G, grad_outputL.size(2), {NM(grad_inputL), NM(grad_inputU)}, {NM(grad_outputL), NM(grad_outputU), NM(posL), NM(posU)}, {NM(grad_weight)});
     Launch L(dev);
     raise_on(ndist_bound_inf_dist_backward_input_weight(F(grad_outputL), F(grad_outputU), I(posL), I(posU),
                                                         grad_outputL.size(0), grad_outputL.size(1),
@@ -221,6 +255,7 @@ void inf_and_bound_forward_nograd(const Tensor& input, const Tensor& inputL, con
     need3d(input, "input"); need3d(output, "output");
     TORCH_CHECK(input.sizes() == inputL.sizes() && input.sizes() == inputU.sizes(), "input and its bounds must have the same shape");
     TORCH_CHECK(output.sizes() == outputL.sizes() && output.sizes() == outputU.sizes(), "the three outputs must have the same shape");
+    agree(input.size(0), output.size(1), input.size(1), G, input.size(2), {NM(input), NM(inputL), NM(inputU)}, {NM(output), NM(outputL), NM(outputU)}, {NM(weight)});
     Launch L(dev);
     raise_on(ndist_inf_and_bound_forward_nograd(F(input), F(inputL), F(inputU), F(weight), input.size(0), output.size(1),
                                                 input.size(1), G, input.size(2), FM(output), FM(outputL), FM(outputU),
@@ -235,6 +270,7 @@ void inf_and_bound_forward(const Tensor& input, const Tensor& inputL, const Tens
                                {"posU", posU, true}});
     need3d(input, "input"); need3d(output, "output");
     TORCH_CHECK(input.sizes() == inputL.sizes() && input.sizes() == inputU.sizes(), "input and its bounds must have the same shape");
+    agree(input.size(0), output.size(1), input.size(1), G, input.size(2), {NM(input), NM(inputL), NM(inputU)}, {NM(output), NM(outputL), NM(outputU), NM(pos), NM(posL), NM(posU)}, {NM(weight)});
     Launch L(dev);
     raise_on(ndist_inf_and_bound_forward(F(input), F(inputL), F(inputU), F(weight), input.size(0), output.size(1),
                                          input.size(1), G, input.size(2), FM(output), IM(pos), FM(outputL), FM(outputU),

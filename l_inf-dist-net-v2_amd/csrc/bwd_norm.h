@@ -67,12 +67,8 @@ __device__ __forceinline__ f16v load_factors(const float* p) {
     typedef const f16v __attribute__((address_space(4))) * cptr;
     return *reinterpret_cast<cptr>(reinterpret_cast<uintptr_t>(p));
 }
-// one factor through the scalar data cache (wave-uniform address)
-__device__ __forceinline__ float load_factor(const float* p) {
-    typedef const float __attribute__((address_space(4))) * cptr;
-    return *reinterpret_cast<cptr>(reinterpret_cast<uintptr_t>(p));
-}
 constexpr int kBwdRowBatch = 16;  // rows whose factors are fetched by one 16-dword scalar load
+
 
 // one (row, co, ci) term for a row slot of the lane, given the wave-uniform factor of that (row, co)
 // R terms (R consecutive row slots of the lane, one co) given the wave-uniform factors of those (row, co) pairs.
@@ -84,14 +80,16 @@ constexpr int kBwdRowBatch = 16;  // rows whose factors are fetched by one 16-dw
 // term carries q * (two roundings) on top of the rounding of t = x - w that no float32 evaluation avoids, which at
 // q = 200 is 1 - 2e-5 relative against the 1e-5 the operator is held to.  Both are known exactly:
 // e = fma(t, a, -v) + t * a_lo is what v is missing (a_lo from the pre-pass, which forms the factor in double
-// precision), and sign(v + e)|v + e|^q = |v|^(q-1) * (v + q e) to first order: three more instructions, used from
-// q = 24 on (-5) and in the rare branch of the skipping variants (`lo` != nullptr).
+// precision), and sign(v + e)|v + e|^q = |v|^(q-1) * (v + q e) to first order: three more instructions (+ 29 % on
+// the kernel), used by the plain variant from q = 64 on (-5).  The skipping variants (-3, -4) evaluate their few
+// surviving terms uncompensated: with the correction inlined into their unrolled bodies the register allocation of
+// the bounds variant went from 48 to 600 - 1000 spilled registers (also with the correction behind a second,
+// rarer test, and as a real call), and both variants lost 35 - 100 % of their speed.
 // The arithmetic is laid out in stages over the R rows: back-to-back dependent vector instructions stall a wave,
 // independent neighbours do not.
 template <int IP, bool WITH_W, int R>
 __device__ __forceinline__ void bwd_terms(const float* __restrict__ xv, float wv, const float (&a)[R], const float (&g2)[R],
-                                          float q, float thr, float* __restrict__ gxa, float (&gwp)[R],
-                                          const float* __restrict__ lo = nullptr) {
+                                          float q, float thr, float* __restrict__ gxa, float (&gwp)[R]) {
     float t[R];
 #pragma unroll
     for (int r = 0; r < R; r++) t[r] = xv[r] - wv;
@@ -138,16 +136,8 @@ __device__ __forceinline__ void bwd_terms(const float* __restrict__ xv, float wv
             for (int r = 0; r < R; r++) {
                 if (hot[r] != 0) {
                     const float e = fast_exp2(q1 * fast_log2(fabsf(t[r])));
-                    float v = t[r];
-                    if (lo != nullptr) {
-                        // what v = fl((x - w) * a) is missing of (x - w) * a_exact; a_lo of this row through the
-                        // scalar cache, only here (wave-uniform address)
-                        const float d = xv[r] - wv;
-                        const float miss = fmaf(d, load_factor(lo + r), fmaf(d, a[r], -v));
-                        v = fmaf(q, miss, v);
-                    }
-                    gxa[r] = fmaf(v, e, gxa[r]);
-                    if (WITH_W) gwp[r] = fmaf(v, e, gwp[r]);
+                    gxa[r] = fmaf(t[r], e, gxa[r]);
+                    if (WITH_W) gwp[r] = fmaf(t[r], e, gwp[r]);
                 }
             }
         }
@@ -460,8 +450,7 @@ __global__ __launch_bounds__(64 * NW, 4) void bwd_fused_kernel(const float* __re
 #pragma unroll
                         for (int r = 0; r < 4; r++)
                             ga[r] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(av), lane0 + q0 + r));
-                        bwd_terms<-3, WITH_W, 4>(&xv[q0], wv, ga, ga, P.q, thr, &gxa[q0], gwp,
-                                                 P.g_off != 0 ? arow + P.g_off + (long)cl * P.Mpad + q0 : nullptr);
+                        bwd_terms<-3, WITH_W, 4>(&xv[q0], wv, ga, ga, P.q, thr, &gxa[q0], gwp);
                     }
                 }
                 if (WITH_W) {
@@ -519,8 +508,7 @@ __global__ __launch_bounds__(64 * NW, 4) void bwd_fused_kernel(const float* __re
                     float ga[RG], gg[RG];
 #pragma unroll
                     for (int r = 0; r < RG; r++) { ga[r] = fa[q0 + r]; gg[r] = fg[q0 + r]; }
-                    bwd_terms<IP, WITH_W, RG>(&xv[bi * RB + q0], wv, ga, gg, P.q, thr, &gxa[bi * RB + q0], gwp,
-                                              IP == -3 && P.g_off != 0 ? ap + P.g_off + q0 : nullptr);
+                    bwd_terms<IP, WITH_W, RG>(&xv[bi * RB + q0], wv, ga, gg, P.q, thr, &gxa[bi * RB + q0], gwp);
                 };
                 // first rows of the batch: their use of the factors is where the wait for the pending request lands
                 group(0);
@@ -639,8 +627,7 @@ __global__ __launch_bounds__(64 * kBwdSmallWaves) void bwd_small_kernel(const fl
                 float ga[RG], gg[RG];
 #pragma unroll
                 for (int r = 0; r < RG; r++) { ga[r] = fa[q0 + r]; gg[r] = fg[q0 + r]; }
-                bwd_terms<IP, WITH_W, RG>(&xv[bi * RB + q0], wv, ga, gg, P.q, thr, &gxa[bi * RB + q0], gwp,
-                                          IP == -3 && P.g_off != 0 ? ap + P.g_off + q0 : nullptr);
+                bwd_terms<IP, WITH_W, RG>(&xv[bi * RB + q0], wv, ga, gg, P.q, thr, &gxa[bi * RB + q0], gwp);
             };
             group(0);
             __builtin_amdgcn_sched_barrier(0);

@@ -268,7 +268,7 @@ __global__ __launch_bounds__(kBoundProbeBlock) void bwd_bound_probe_kernel(const
 constexpr int kBwdTransposeMinHW = 16;
 
 // What the launcher decides from the shape and the exponent alone.
-constexpr float kBwdCompensateFromQ = 24.0f;
+constexpr float kBwdCompensateFromQ = 64.0f;
 struct BwdPlan {
     int ip;              // exponent variant of the kernels
     bool second;         // the variant reads a second factor array
@@ -357,7 +357,7 @@ int launch_norm_backward(const float* gout, const float* x, const float* w, cons
     if (!rc) {
         dim3 grid(ceil_div(P.Mpad, 32), ceil_div(s.COg * s.G, 32));
         hipLaunchKernelGGL(bwd_prepare_kernel, grid, dim3(256), 0, st, out, gout, aT, s, P.Mpad, q, P.g_off,
-                           ip == -2 ? 1 : (ip == -5 ? 2 : 0), adaptive ? aux + 4 : (float*)nullptr);
+                           ip == -2 ? 1 : (pl.second ? 2 : 0), adaptive ? aux + 4 : (float*)nullptr);
         if (hip_failed(hipGetLastError())) rc = 4;
     }
     const long nx = (long)s.M * s.CIg * s.G;

@@ -27,11 +27,24 @@ int hip_status(hipError_t e) {
     return NDIST_ERR_HIP;
 }
 
+namespace {
+constexpr int kMaxDev = 64;
+DeviceInfo g_di_cache[kMaxDev];
+bool g_di_have[kMaxDev] = {};
+std::mutex g_di_mu;
+}  // namespace
+
+bool device_info_cached() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) dev = 0;
+    std::lock_guard<std::mutex> lock(g_di_mu);
+    return g_di_have[dev];
+}
+
 const DeviceInfo& device_info() {
-    constexpr int kMaxDev = 64;
-    static DeviceInfo cache[kMaxDev];
-    static bool have[kMaxDev] = {};
-    static std::mutex mu;
+    DeviceInfo* cache = g_di_cache;
+    bool* have = g_di_have;
+    std::mutex& mu = g_di_mu;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) dev = 0;
     std::lock_guard<std::mutex> lock(mu);
@@ -150,6 +163,14 @@ void ndist_set_profiling(int enable) { g_profiling.store(enable ? 1 : 0); }
 void ndist_set_skip_mode(int skip, int bounds) { set_skip_mode(skip, bounds); }
 void ndist_set_hot_mode(int mode) { set_hot_mode(mode); }
 void ndist_set_scaled_mode(int mode) { set_scaled_mode(mode); }
+void ndist_get_modes(int* skip, int* bounds, int* hot, int* scaled) {
+    int s = -1, b = -1;
+    get_skip_mode(&s, &b);
+    if (skip != nullptr) *skip = s;
+    if (bounds != nullptr) *bounds = b;
+    if (hot != nullptr) *hot = hot_mode();
+    if (scaled != nullptr) *scaled = scaled_mode();
+}
 
 int ndist_release_scratch(void) { return scratch_release_all(); }
 
@@ -161,6 +182,13 @@ void ndist_scratch_counters(long* mallocs, long* frees) {
 }
 
 size_t ndist_noalloc_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int ndist_noalloc_prepare(void) {
+    char* base = nullptr;
+    if (int rc = hip_status(static_scratch_base(&base, true))) return rc;
+    (void)device_info();
+    return device_info_cached() ? NDIST_OK : NDIST_ERR_NO_DEVICE;
+}
 
 int ndist_last_kernel_ms(float* ms) {
     if (ms == nullptr) return NDIST_ERR_NULL_POINTER;
@@ -222,7 +250,13 @@ int ndist_norm_dist_backward_input_weight_noalloc(const float* grad_output, cons
     if (int rc = make_geom(B, CO, CI, G, HW, &s)) return rc;
     // the factor array is the one piece of scratch the kernels cannot do without: refuse before anything is launched
     if (norm_backward_scratch_bytes(s, p) > kStaticScratchBytes) return NDIST_ERR_TOO_LARGE;
-    StaticScratchScope scope;  // scratch_alloc serves from the fixed array while this lives; looks its address up once
+    // scratch_alloc serves from the fixed array while the scope lives.  The array's address and the device's
+    // properties are looked up once per device: by ndist_noalloc_prepare() or by the first call outside a capture;
+    // a call on a capturing stream that finds them missing refuses instead of querying the runtime mid-capture.
+    const bool capturing = stream_is_capturing((hipStream_t)stream);
+    if (capturing && !device_info_cached()) return NDIST_ERR_CAPTURE;
+    StaticScratchScope scope(!capturing);
+    if (scope.status == hipErrorStreamCaptureUnsupported) return NDIST_ERR_CAPTURE;
     if (int rc = hip_status(scope.status)) return rc;
     return launch_norm_backward(grad_output, input, weight, output, s, grad_input, grad_weight, p, (hipStream_t)stream);
 }

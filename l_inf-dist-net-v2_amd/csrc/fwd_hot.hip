@@ -593,12 +593,13 @@ int env_hot_mode() {
     const char* v = getenv("NORM_DIST_HOT");
     return v == nullptr || v[0] < '0' || v[0] > '3' ? -1 : v[0] - '0';
 }
-std::atomic<int> g_hot_mode{env_hot_mode()};
+const int g_env_hot = env_hot_mode();
+thread_local int t_hot_mode = g_env_hot;  // per calling host thread, like the other overrides
 
 }  // namespace
 
-void set_hot_mode(int mode) { g_hot_mode.store(mode < 0 || mode > 3 ? -1 : mode); }
-int hot_mode() { return g_hot_mode.load(); }
+void set_hot_mode(int mode) { t_hot_mode = mode < 0 || mode > 3 ? g_env_hot : mode; }
+int hot_mode() { return t_hot_mode; }
 
 static int plan_blocks(const Geom& s) {
     return (int)(((long)s.M * s.G + (long)s.COg * s.G + kPlanRows - 1) / kPlanRows);

@@ -452,15 +452,22 @@ static int env_mode(const char* name) {
     const char* v = getenv(name);
     return v == nullptr ? -1 : (v[0] == '0' ? 0 : 1);
 }
-static std::atomic<int> g_skip_mode{env_mode("NORM_DIST_SKIP")}, g_bounds_mode{env_mode("NORM_DIST_BWD_BOUNDS")};
+// The overrides belong to the calling host thread (thread_local): a thread that never called the setter uses the
+// value the environment gave at load time, and no thread can leave another one on a different kernel path.
+static const int g_env_skip = env_mode("NORM_DIST_SKIP"), g_env_bounds = env_mode("NORM_DIST_BWD_BOUNDS");
+static thread_local int t_skip_mode = g_env_skip, t_bounds_mode = g_env_bounds;
 void set_skip_mode(int skip, int bounds) {
-    g_skip_mode.store(skip < 0 ? -1 : (skip ? 1 : 0));
-    g_bounds_mode.store(bounds < 0 ? -1 : (bounds ? 1 : 0));
+    t_skip_mode = skip < 0 ? g_env_skip : (skip ? 1 : 0);
+    t_bounds_mode = bounds < 0 ? g_env_bounds : (bounds ? 1 : 0);
+}
+void get_skip_mode(int* skip, int* bounds) {
+    *skip = t_skip_mode;
+    *bounds = t_bounds_mode;
 }
 static int override_limit(int mode, int probed_limit) { return mode < 0 ? probed_limit : (mode == 0 ? 0 : 0x7fffffff); }
-int skip_override_limit(int probed_limit) { return override_limit(g_skip_mode.load(), probed_limit); }
-int bounds_override_limit(int probed_limit) { return override_limit(g_bounds_mode.load(), probed_limit); }
-bool skip_forced_on() { return g_skip_mode.load() == 1; }
+int skip_override_limit(int probed_limit) { return override_limit(t_skip_mode, probed_limit); }
+int bounds_override_limit(int probed_limit) { return override_limit(t_bounds_mode, probed_limit); }
+bool skip_forced_on() { return t_skip_mode == 1; }
 
 // ---- one-pass normalised sum with a per-row scale (OpRowScaled) ------------------------------------------
 
@@ -536,13 +543,15 @@ __global__ __launch_bounds__(256) void norm_fixup_kernel(const float* __restrict
     }
 }
 
-static std::atomic<int> g_scaled_mode{env_mode("NORM_DIST_ROW_SCALE")};
-void set_scaled_mode(int mode) { g_scaled_mode.store(mode < 0 ? -1 : (mode ? 1 : 0)); }
+static const int g_env_scaled = env_mode("NORM_DIST_ROW_SCALE");
+static thread_local int t_scaled_mode = g_env_scaled;
+void set_scaled_mode(int mode) { t_scaled_mode = mode < 0 ? g_env_scaled : (mode ? 1 : 0); }
+int scaled_mode() { return t_scaled_mode; }
 // Up to p = 48 a scale 3.2 times the true maximum still keeps the sum above 2^-90; beyond, too many outputs would
 // take the slow exact route on ordinary data.
 constexpr float kMaxRowScaledP = 48.0f;
 static bool row_scaled_applies(const Geom& s, float p) {
-    const int mode = g_scaled_mode.load();
+    const int mode = t_scaled_mode;
     if (mode == 0 || s.HW != 1 || !(p <= kMaxRowScaledP) || skinny_applies(s)) return false;
     return mode == 1 || (double)s.M * s.COg * s.G * s.CIg >= 2e7;
 }

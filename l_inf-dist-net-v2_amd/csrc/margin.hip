@@ -65,9 +65,12 @@ __global__ __launch_bounds__(1024) void hinge_forward_kernel(const float* __rest
         float best = 0.f, rs = 0.f;
         int at = -1;
         for (int c = 0; c < C; c++) {
-            const float r = fmaxf(margin[(long)b * C + c], 0.f);
+            // relu that lets NaN through, and a maximum that NaN wins, as torch's clamp(min=0) and max do in the
+            // reference's loss: diverged activations or the NaN row of an out-of-range label must reach the loss
+            const float m = margin[(long)b * C + c];
+            const float r = m > 0.f ? m : (m != m ? m : 0.f);
             rs += r;
-            if (r > best) { best = r; at = c; }
+            if (r > best || (r != r && best == best)) { best = r; at = c; }
         }
         argmax[b] = at;
         smax += best;

@@ -50,6 +50,7 @@ struct DeviceInfo {
 };
 // Properties of the current device, queried once per device and cached.
 const DeviceInfo& device_info();
+bool device_info_cached();  // the current device's properties have been queried already
 
 // Records a failing HIP call for ndist_last_hip_error(); returns true when `e` is an error.
 bool hip_failed(hipError_t e);
@@ -87,7 +88,7 @@ bool stream_is_capturing(hipStream_t st);
 // array and race.
 constexpr size_t kStaticScratchBytes = 24u << 20;
 struct StaticScratchScope {
-    StaticScratchScope();
+    explicit StaticScratchScope(bool may_query = true);  // false: never look the array's address up (capture)
     ~StaticScratchScope();
     StaticScratchScope(const StaticScratchScope&) = delete;
     StaticScratchScope& operator=(const StaticScratchScope&) = delete;
@@ -97,6 +98,7 @@ struct StaticScratchScope {
     int live;
 };
 bool static_scratch_active();
+hipError_t static_scratch_base(char** out, bool may_query);
 
 // Seeds and k-tile bounds for the forward operators that skip whole k-tiles (fully-connected layout, HW == 1).
 //   seed    [M][COg*G] as the output: for every output, the larger of the two pairs |x - w| at the k where its x row
@@ -269,9 +271,11 @@ int skip_override_limit(int probed_limit);
 bool skip_forced_on();
 int bounds_override_limit(int probed_limit);
 void set_skip_mode(int skip, int bounds);
+void get_skip_mode(int* skip, int* bounds);  // the calling thread's current values
 // Tuning and test aid (ndist_set_scaled_mode / NORM_DIST_ROW_SCALE): the one-pass normalised forward for
 // 10 < p <= 48 in the fully connected layout; -1 from 2e7 pairs on (default), 0 never, 1 whenever the layout allows.
 void set_scaled_mode(int mode);
+int scaled_mode();
 int launch_unfold(const float* x, const UnfoldGeom& u, float* out, hipStream_t st);
 int launch_fold(const float* gout, const UnfoldGeom& u, float* gx, hipStream_t st);
 // the patches as rows [B * OH * OW][C * kh * kw] (the transpose of the unfolded tensor); -1: geometry not served

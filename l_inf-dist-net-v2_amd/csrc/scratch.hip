@@ -120,7 +120,9 @@ bool stream_is_capturing(hipStream_t st) {
     return cs != hipStreamCaptureStatusNone;
 }
 
-hipError_t static_scratch_base(char** out) {
+// may_query == false (the stream is being captured): only an address that an earlier call has already looked up
+// is returned; the lookup itself is not made from inside a capture
+hipError_t static_scratch_base(char** out, bool may_query) {
     constexpr int kMaxDev = 64;
     static char* base[kMaxDev] = {};
     static std::mutex mu;
@@ -129,6 +131,7 @@ hipError_t static_scratch_base(char** out) {
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= kMaxDev) return hipErrorInvalidDevice;
     std::lock_guard<std::mutex> lock(mu);
+    if (base[dev] == nullptr && !may_query) return hipErrorStreamCaptureUnsupported;
     if (base[dev] == nullptr) {
         // once per device, with that device current: every device holds its own copy of the array
         char* ptr = nullptr;
@@ -141,8 +144,8 @@ hipError_t static_scratch_base(char** out) {
     return hipSuccess;
 }
 
-StaticScratchScope::StaticScratchScope() : status(hipSuccess), base(nullptr), used(0), live(0) {
-    status = static_scratch_base(&base);
+StaticScratchScope::StaticScratchScope(bool may_query) : status(hipSuccess), base(nullptr), used(0), live(0) {
+    status = static_scratch_base(&base, may_query);
     if (status == hipSuccess) t_static = this;
 }
 StaticScratchScope::~StaticScratchScope() {

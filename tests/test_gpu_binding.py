@@ -39,6 +39,25 @@ _C.bound_inf_dist_forward_nograd(x - 0.1, x + 0.1, w, yl, yu, 1); res["bound"] =
 img = torch.randn(2, 4, 8, 8, generator=gen).cuda(); cw = torch.randn(6, 36, generator=gen).cuda()
 co = torch.empty(2, 6, 64, device="cuda")
 _C.conv_inf_dist_forward_nograd(img, cw, co, 1, 3, 1, 1, 1); res["conv"] = digest(co)
+# tensors whose sizes do not agree are refused on the host (a kernel would index them out of bounds)
+def refused(fn, *a):
+    try:
+        fn(*a)
+    except RuntimeError:
+        return True
+    return False
+short_w = w[:CO - 1].contiguous(); narrow_w = w[:, :CI - 8].contiguous(); small_out = out[:, :CO - 1].contiguous()
+res["refusals"] = [
+    refused(_C.inf_dist_forward_nograd, x, short_w, out, 1),
+    refused(_C.inf_dist_forward_nograd, x, narrow_w, out, 1),
+    refused(_C.inf_dist_forward, x, w, out, pos[:, :CO - 1].contiguous(), 1),
+    refused(_C.norm_dist_forward, x, w, out, 3, 8.0),
+    refused(_C.norm_dist_backward_input_weight, g, x, w, small_out, gx, gw, 1, 8.0),
+    refused(_C.norm_dist_backward_input_weight, g, x, w, out, gx[:B - 1].contiguous(), gw, 1, 8.0),
+    refused(_C.norm_dist_backward_input_weight, g, x, w, out, gx, gw[:CO - 1].contiguous(), 1, 8.0),
+    refused(_C.inf_dist_backward_input_weight, g, pos, gx, gw[:CO - 1].contiguous(), 1),
+    refused(_C.bound_inf_dist_forward_nograd, x - 0.1, (x + 0.1)[:B - 1].contiguous(), w, yl, yu, 1),
+]
 # host cost of queueing one small call (the device is kept busy by the calls themselves)
 xs, ws, os_ = x[:8].contiguous(), w[:16].contiguous(), torch.empty(8, 16, 1, device="cuda")
 for _ in range(200): _C.inf_dist_forward_nograd(xs, ws, os_, 1)
@@ -72,6 +91,7 @@ def test_both_bindings_give_the_same_bits():
     for k in ("inf_fwd", "p8_fwd", "p8_bwd_gw", "bound", "conv"):
         assert ext[k] == ct[k], k
     assert abs(ext["inf_bwd_sum"] - ct["inf_bwd_sum"]) < 1e-3
+    assert all(ext["refusals"]) and all(ct["refusals"]), (ext["refusals"], ct["refusals"])  # mismatched sizes
     print("host microseconds per queued call: extension %.1f, ctypes %.1f" % (ext["host_us_per_call"], ct["host_us_per_call"]))
     assert ext["host_us_per_call"] < 3 * ct["host_us_per_call"] + 20  # sanity only: neither route may stall
 
@@ -88,7 +108,7 @@ def test_extension_checks_like_the_reference_binding():
         E.inf_dist_forward_nograd(torch.randn(4, 16, 1, device="cuda")[:, ::2], w, out, 1)
     with pytest.raises(RuntimeError, match="dtype"):
         E.inf_dist_forward_nograd(x.double(), w, out, 1)
-    with pytest.raises(RuntimeError, match="status 2"):  # CI not divisible by G
+    with pytest.raises(RuntimeError, match="groups"):  # CI not divisible by G
         E.inf_dist_forward_nograd(x, w, out, 3)
     with pytest.raises(RuntimeError, match="status 3"):
         E.norm_dist_forward(x, w, out, 1, -1.0)

@@ -153,12 +153,12 @@ def test_backward_large_p_probe_and_skipping(dist, p):
     # fp32 evaluation agrees with the float64 oracle to better than about 1e-7 * p on the large elements: the
     # tolerance is 1e-5, or twice the error of a plain float32 evaluation of the same terms where that misses 1e-5
     ex, _ = O.norm_dist_backward(g[rows], x[rows], w, out[rows], p, with_weight=False)
-    tol, _ = backward_tolerances(g[rows], x[rows], w, out[rows], p, 1, ex, None)
+    tol, _ = backward_tolerances(g[rows], x[rows], w, out[rows], p, 1, ex, None, skipping=True)
     assert_close(gx[rows], ex, tol=tol, what="grad_input rows %s p=%g" % (dist, p))
-    tol5, _ = backward_tolerances(g[5:6], x[5:6], w, out[5:6], p, 1, ex[1:2], None)
-    assert_close(gx[5:6], ex[1:2], tol=tol5, what="grad_input of the row with small grad_output")
+    # (one row: the comparison rests on a few elements, so the bound is that of the four rows together)
+    assert_close(gx[5:6], ex[1:2], tol=2 * tol, what="grad_input of the row with small grad_output")
     _, ew = O.norm_dist_backward(g[:, cols], x, w[cols], out[:, cols], p)
-    _, tol = backward_tolerances(g[:, cols], x, w[cols], out[:, cols], p, 1, None, ew)
+    _, tol = backward_tolerances(g[:, cols], x, w[cols], out[:, cols], p, 1, None, ew, skipping=True)
     assert_close(gw[cols], ew, tol=tol, what="grad_weight columns %s p=%g" % (dist, p))
 
 

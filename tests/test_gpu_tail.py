@@ -80,3 +80,28 @@ def test_label_outside_the_classes_gives_nan_rows_not_a_fault():
     gx = torch.full_like(x, 7.0)
     _C.margin_backward(torch.ones_like(x), t, 0.1, gx, None, None)
     assert torch.isfinite(gx).all()
+
+
+def test_nan_margins_reach_the_loss_as_in_the_torch_formula():
+    """clamp(min=0).max().mean() of the reference's loss (main.py:304-310) propagates NaN: a NaN margin (diverged
+    activations, the NaN row of an out-of-range label) must give a NaN loss, not a finite one; the gradient of the
+    NaN entries is what torch's clamp / max backward give them."""
+    from core.norm_dist import hinge_loss
+    torch.manual_seed(7)
+    margin = torch.randn(12, 10, device="cuda")
+    margin[3, 4] = float("nan")
+    margin[8] = float("nan")
+    for mix in (0.25, 0.0, 1.0):
+        a = margin.clone().requires_grad_(True)
+        b = margin.clone().requires_grad_(True)
+        loss = hinge_loss(a, mix)
+        res = b.clamp(min=0)
+        want = (1 - mix) * res.max(dim=1)[0].mean() + mix * res.mean()
+        assert torch.isnan(loss) and torch.isnan(want)
+        loss.backward()
+        want.backward()
+        assert torch.equal(torch.isnan(a.grad), torch.isnan(b.grad))
+        # finite everywhere else, and zero on the NaN entries themselves (masked by relu's derivative)
+        assert torch.isfinite(a.grad).all() and float(a.grad[8].abs().sum()) == 0.0 and float(a.grad[3, 4]) == 0.0
+    clean = torch.randn(12, 10, device="cuda")
+    assert torch.isfinite(hinge_loss(clean, 0.25))

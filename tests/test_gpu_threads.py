@@ -50,3 +50,34 @@ def test_concurrent_callers_on_their_own_streams(p):
             # float atomics: the order of summation may differ from run to run, also without threads
             assert float((gx - gx0).abs().max()) <= 1e-5 * float(gx0.abs().max())
             assert float((gw - gw0).abs().max()) <= 1e-5 * float(gw0.abs().max())
+
+
+def test_mode_overrides_belong_to_the_calling_thread():
+    """ndist_set_skip_mode / hot_mode / scaled_mode change the calling thread's settings only: a thread that forces
+    kernel variants (a test, a tuning run) cannot leave other callers on another kernel path."""
+    from core import _C
+    base = _C.get_modes()
+    seen = {}
+
+    def other():
+        seen["before"] = _C.get_modes()
+        _C.set_skip_mode(1, 0)
+        _C.set_hot_mode(3)
+        _C.set_scaled_mode(0)
+        seen["after"] = _C.get_modes()
+
+    t = threading.Thread(target=other)
+    t.start()
+    t.join(30)
+    assert seen["before"] == base and seen["after"] == (1, 0, 3, 0)
+    assert _C.get_modes() == base                      # untouched here
+    _C.set_hot_mode(2)
+    try:
+        assert _C.get_modes()[2] == 2
+        t = threading.Thread(target=lambda: seen.__setitem__("fresh", _C.get_modes()))
+        t.start()
+        t.join(30)
+        assert seen["fresh"] == base                   # a new thread starts from the environment's values
+    finally:
+        _C.set_hot_mode(-1)
+    assert _C.get_modes() == base

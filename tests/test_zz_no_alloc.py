@@ -1,7 +1,8 @@
 """The entry point that allocates nothing (ndist_norm_dist_backward_input_weight_noalloc, no counterpart in the
 reference): called through the C ABI, checked against the allocating entry point it is a variant of (bit for bit
 where that path sums in a fixed order, to 1e-5 where it uses atomics) and against the float64 oracle, on two calls in a
-row, the second with a smaller input; the library's own allocation counters must not move across the calls."""
+row, the second with a smaller input; the library's own allocation counters must not move across the calls; and
+recorded into a HIP graph, which is what such callers do with it."""
 import numpy as np
 import pytest
 import torch
@@ -86,3 +87,39 @@ def test_headline_shape_fits_and_larger_is_refused():
     assert e.value.status == _C.ERR_TOO_LARGE
     torch.cuda.synchronize()
     assert float(gx.min()) == 7.0 and float(gw.min()) == 7.0  # untouched
+
+
+def test_captured_into_a_graph_and_replayed():
+    """One call of the no-allocation entry point recorded into a HIP graph (its whole purpose), replayed several
+    times with eager work and synchronisations in between; every replay is compared with the allocating entry
+    point on the inputs the replay saw.  A capture that starts before the array's address is known is refused."""
+    from core import _C
+    assert _C._lib.ndist_noalloc_prepare() == 0
+    x, w, g = _inputs(11, 300, 200, 520)
+    xt, wt, gt = (torch.from_numpy(a).cuda() for a in (x, w, g))
+    out = torch.empty(300, 200, 1, device="cuda")
+    gx, gw = torch.full_like(xt, float("nan")), torch.full_like(wt, float("nan"))
+    _C.norm_dist_forward(xt, wt, out, 1, 8.0)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    print("capturing", flush=True)
+    with torch.cuda.graph(graph):
+        _C.norm_dist_backward_input_weight_noalloc(gt, xt, wt, out, gx, gw, 1, 8.0)
+    torch.cuda.synchronize()
+    for it in range(3):
+        print("replay", it, flush=True)
+        if it:  # new inputs in the captured buffers, written by eager work between the replays
+            xt.copy_(torch.from_numpy(_inputs(20 + it, 300, 200, 520)[0]).cuda())
+            gt.mul_(-0.5)
+            _C.norm_dist_forward(xt, wt, out, 1, 8.0)
+        gx.fill_(float("nan"))
+        gw.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        rx, rw = torch.empty_like(xt), torch.empty_like(wt)
+        _C.norm_dist_backward_input_weight(gt, xt, wt, out, rx, rw, 1, 8.0)
+        torch.cuda.synchronize()
+        assert_close(gx.cpu().numpy(), rx.cpu().numpy(), tol=REL, what="replay %d grad_input" % it)
+        assert_close(gw.cpu().numpy(), rw.cpu().numpy(), tol=REL, what="replay %d grad_weight" % it)
+    del graph
