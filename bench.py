@@ -133,7 +133,20 @@ def other_workloads(torch, _C, xd, wd, gd):
         o5 = out.clone()
         res["p%g_backward_unit_weights_b512_5120x5120" % pp] = tm(
             lambda: _C.norm_dist_backward_input_weight(gd, xd, w1, o5, gx, gw, 1, pp))
-    del w1
+    # the max-reductions on the same dense data (nothing to skip: behind the hot-tile plan the plain tiled kernel
+    # runs), next to the library's own plain path with all data-dependent skipping switched off
+    pos1 = torch.empty(B, CO, 1, device=dev, dtype=torch.int32)
+    xl1, xu1 = xd - 8 / 255, xd + 8 / 255
+    yl1, yu1, pu1 = torch.empty_like(out), torch.empty_like(out), torch.empty_like(pos1)
+    for tag, skip in (("", -1), ("_skip_off", 0)):
+        _C.set_skip_mode(skip, -1)
+        try:
+            res["pinf_forward_unit_weights%s_b512_5120x5120" % tag] = tm(lambda: _C.inf_dist_forward(xd, w1, out, pos1, 1))
+            res["ibp_bounds_forward_unit_weights%s_b512_5120x5120" % tag] = tm(
+                lambda: _C.bound_inf_dist_forward(xl1, xu1, w1, yl1, yu1, pos1, pu1, 1))
+        finally:
+            _C.set_skip_mode(-1, -1)
+    del w1, pos1, xl1, xu1, yl1, yu1, pu1
     # small batch (64 rows): bound by streaming w (105 MB) rather than by arithmetic
     xs, gs = xd[:64].contiguous(), gd[:64].contiguous()
     outs = torch.empty(64, CO, 1, device=dev)

@@ -227,13 +227,29 @@ int launch_bound_forward(const float* xl, const float* xu, const float* w, const
         if ((bounded || hot) && front == nullptr && hip_failed(scratch_free(scratch, st)) && !rc) rc = 4;
         return rc;
     };
+    // two dense candidates behind the hot-tile plan, as in launch_inf_forward
+    const bool two = bounded && hot && gate != nullptr;
+    FwdParams Q = P;  // the plain candidate
+    if (two) {
+        P.gate = gate + 4;
+        Q.gate = gate + 5;
+        Q.aux = Q.aux2 = nullptr;
+        Q.tile_x = Q.tile_w = nullptr;
+    }
     if (pl == nullptr) {
-        return done(bounded ? launch_fwd<OpBound<false, true>, CfgBoundT, CfgMid, CfgSmall>(P, st)
-                            : launch_fwd_conv<OpBound<false>, CfgBoundN, CfgMid, CfgSmall>(P, st));
+        int rc = bounded ? launch_fwd<OpBound<false, true>, CfgBoundT, CfgMid, CfgSmall>(P, st)
+                         : launch_fwd_conv<OpBound<false>, CfgBoundN, CfgMid, CfgSmall>(P, st);
+        if (!rc && two) rc = launch_fwd_conv<OpBound<false>, CfgBoundN, CfgMid, CfgSmall>(Q, st);
+        return done(rc);
     }
     int kt = 0;
-    const int rc = bounded ? launch_fwd_layouts<false, OpBound<true, true>, CfgBoundT, CfgSmall>(P, st, &kt)
-                           : launch_fwd_layouts<true, OpBound<true>, CfgBoundT, CfgSmall>(P, st, &kt);
+    int rc = bounded ? launch_fwd_layouts<false, OpBound<true, true>, CfgBoundT, CfgSmall>(P, st, &kt)
+                     : launch_fwd_layouts<true, OpBound<true>, CfgBoundT, CfgSmall>(P, st, &kt);
+    if (!rc && two) {
+        int kt2 = 0;
+        rc = launch_fwd_layouts<true, OpBound<true>, CfgBoundT, CfgSmall>(Q, st, &kt2);
+        if (!rc && kt2 != kt) rc = 2;  // (same candidate list and cost model: cannot differ)
+    }
     if (rc) return done(rc);
     const int imp = cv != nullptr;
     if (rescan_sorted_applies(s, kt)) {

@@ -80,7 +80,8 @@ __device__ __forceinline__ void hot_group_maxima(const float* __restrict__ seed_
 // t of a row's mask = tile t is hot (a row's record: one word naming its non-zero mask words, then the mask words).
 // The workgroups leave their counts of hot (row, tile) entries per side in
 // `partial`; the last one to finish (a ticket in dec[3], cleared by the row pre-pass) adds them up and decides:
-//   dec[0] = 1: the rows of x select the tiles, 2: the rows of w, 0: too many hot tiles, the dense kernels run.
+//   dec[0] = 1: the rows of x select the tiles, 2: the rows of w, 0: too many hot tiles, the dense kernels run
+//   (dec[4] / dec[5] then say which of them, see below).
 // Cost of a side = its hot entries x the length of the other side.  mode: 1 always the cheaper side, 2 / 3 always
 // the x / w side, else the cheaper side if it touches at most 1 / frac of all (row, column, tile) triples.
 constexpr int kPlanRows = 64, kPlanRowsPerWave = kPlanRows / 16;
@@ -100,7 +101,7 @@ struct PlanJob {
 __global__ __launch_bounds__(1024) void hot_plan_kernel(const PlanJob ja, const PlanJob jb, int nblk,
                                                         const float* __restrict__ seed_w,
                                                         const float* __restrict__ tile_w, const Geom s, int ntile,
-                                                        int nword, int mode, int frac) {
+                                                        int nword, int mode, int frac, int dense_ok) {
     const bool second = (int)blockIdx.x >= nblk;
     const PlanJob& job = second ? jb : ja;
     const int bid = (int)blockIdx.x - (second ? nblk : 0);
@@ -230,6 +231,13 @@ __global__ __launch_bounds__(1024) void hot_plan_kernel(const PlanJob ja, const 
         else if (mode == 3) choice = 2;
         else if (mode != 1 && (costx <= costw ? costx : costw) * frac > total) choice = 0;
         dec[0] = choice;
+        // Which of the two dense kernels runs when the hot tiles do not: with (nearly) every tile hot on both sides
+        // under the separable test, the kernel that checks tile bounds has nothing to drop and only pays for its
+        // bounds, votes and flags (a third per stage): the plain tiled kernel takes over.  Gate words, 0 = run.
+        const bool dense = dense_ok != 0 && tot[0] * 10 > (long long)s.M * s.G * ntile * 9 &&
+                           tot[1] * 10 > (long long)s.COg * s.G * ntile * 9;
+        dec[4] = choice != 0 || dense ? 1 : 0;   // tile-skipping kernel (and the output seeds it starts from)
+        dec[5] = choice != 0 || !dense ? 1 : 0;  // plain kernel
         dec[1] = (int)(tot[0] > 0x7fffffff ? 0x7fffffff : tot[0]);  // for inspection
         dec[2] = (int)(tot[1] > 0x7fffffff ? 0x7fffffff : tot[1]);
     }
@@ -501,7 +509,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(P::kMinWave
     uint32_t (*tc)[kHotRows][17] = reinterpret_cast<uint32_t (*)[kHotRows][17]>(lds + NF * kHotRows * 17);
     const int choice = dec[0];
     if (choice == 0) {
-        if (blockIdx.x < seed_blocks) P::seed_outputs(x, x2off, w, s, seeds, blockIdx.x, lds);
+        if (dec[4] == 0 && blockIdx.x < seed_blocks) P::seed_outputs(x, x2off, w, s, seeds, blockIdx.x, lds);
         return;
     }
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -614,7 +622,8 @@ size_t hot_scratch_floats(const Geom& s) {
 
 // Where the plan's results lie in an operator's hot scratch (`base`).
 struct HotLayout {
-    int* dec;  // [0] decision, [1], [2] hot entries per side, [3] ticket (cleared by the row pre-pass)
+    int* dec;  // [0] decision, [1], [2] hot entries per side, [3] ticket (cleared by the row pre-pass), [4], [5] gate
+               // words of the two dense kernels (0 = run)
     int* partial;
     uint32_t* mask_x;
     uint32_t* mask_w;
@@ -643,7 +652,7 @@ int launch_joint_hot_plan(const Geom& s, const SeedBuffers& sb, float* base, con
     const HotLayout ha = hot_layout(s, sb, base), hb = hot_layout(s, sb_box, base_box);
     hipLaunchKernelGGL(hot_plan_kernel, dim3(2 * ha.nblk), dim3(1024), 2 * s.G * sizeof(unsigned), st,
                        plan_job(ha, sb, false), plan_job(hb, sb_box, true), ha.nblk, sb.seed_w, sb.tile_w, s, sb.ntile,
-                       ha.nword, hot_mode(), kHotFraction);
+                       ha.nword, hot_mode(), kHotFraction, skip_forced_on() ? 0 : 1);
     return hip_failed(hipGetLastError()) ? 4 : 0;
 }
 
@@ -660,7 +669,7 @@ static int launch_hot(const float* x, const float* x2, const float* w, const Geo
     if (!plan_done) {
         const PlanJob job = plan_job(h, sb, x2 != nullptr);
         hipLaunchKernelGGL(hot_plan_kernel, dim3(h.nblk), dim3(1024), 2 * s.G * sizeof(unsigned), st, job, job, h.nblk,
-                           sb.seed_w, sb.tile_w, s, sb.ntile, nword, hot_mode(), kHotFraction);
+                           sb.seed_w, sb.tile_w, s, sb.ntile, nword, hot_mode(), kHotFraction, skip_forced_on() ? 0 : 1);
     }
     int vec = s.CIg % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0;
     if (x2 != nullptr) vec = vec && (uintptr_t)x2 % 16 == 0;

@@ -215,13 +215,31 @@ int launch_inf_forward(const float* x, const float* w, const Geom& s, float* out
         if ((bounded || hot) && front == nullptr && hip_failed(scratch_free(scratch, st)) && !rc) rc = 4;
         return rc;
     };
+    // With the hot-tile plan ahead there are two dense candidates behind it: the kernel that drops k-tiles by their
+    // bounds, and, for data on which the plan found (nearly) every tile hot, the plain kernel (gate words 4 and 5 of
+    // the plan's decision; both leave the winning k-tile in pos, in the same configuration).
+    const bool two = bounded && hot && gate != nullptr;
+    FwdParams Q = P;  // the plain candidate
+    if (two) {
+        P.gate = gate + 4;
+        Q.gate = gate + 5;
+        Q.aux = nullptr;
+        Q.tile_x = Q.tile_w = nullptr;
+    }
     if (pos == nullptr) {
-        return done(bounded ? launch_fwd<OpInf<false, true>, CfgWideT, CfgMid, CfgSmall>(P, st)
-                            : launch_fwd_conv<OpInf<false>, CfgWide4, CfgBig, CfgSmall, CfgWide>(P, st));
+        int rc = bounded ? launch_fwd<OpInf<false, true>, CfgWideT, CfgMid, CfgSmall>(P, st)
+                         : launch_fwd_conv<OpInf<false>, CfgWide4, CfgBig, CfgSmall, CfgWide>(P, st);
+        if (!rc && two) rc = launch_fwd_conv<OpInf<false>, CfgWide4, CfgBig, CfgSmall, CfgWide>(Q, st);
+        return done(rc);
     }
     int kt = 0;
-    const int rc = bounded ? launch_fwd_layouts<false, OpInf<true, true>, CfgWideT, CfgMid, CfgSmall>(P, st, &kt)
-                           : launch_fwd_layouts<true, OpInf<true>, CfgWideT, CfgMid, CfgSmall>(P, st, &kt);
+    int rc = bounded ? launch_fwd_layouts<false, OpInf<true, true>, CfgWideT, CfgMid, CfgSmall>(P, st, &kt)
+                     : launch_fwd_layouts<true, OpInf<true>, CfgWideT, CfgMid, CfgSmall>(P, st, &kt);
+    if (!rc && two) {
+        int kt2 = 0;
+        rc = launch_fwd_layouts<true, OpInf<true>, CfgWideT, CfgMid, CfgSmall>(Q, st, &kt2);
+        if (!rc && kt2 != kt) rc = 2;  // (same candidate list and cost model: cannot differ)
+    }
     if (rc) return done(rc);
     if (rescan_sorted_applies(s, kt))
         return done(launch_rescan_sorted<0>(x, nullptr, w, out, pos, s, kt, st, cv ? &pm : nullptr));

@@ -174,3 +174,29 @@ def test_long_reductions_where_little_can_be_dropped(modes, kind):
         got = gpu_bound_forward(xl, xu, w, with_pos=with_pos)
         for e, v in zip(expect, got):
             assert v is None or np.array_equal(e, v), "interval bounds " + kind
+
+
+@pytest.mark.parametrize("kind", ["normal", "small_w", "diagonal", "mixed"])
+def test_unforced_routes_at_a_size_where_all_three_are_queued(kind):
+    """Nothing forced, a problem large enough for the hot-tile plan and both dense kernels behind it: dense data
+    (`normal`: every tile hot on both sides, the plain tiled kernel runs), sparse data (the hot tiles run) and
+    `mixed` data (a quarter of the rows of x carry outliers: too many hot tiles for the hot-tile kernel, few enough
+    for the tile-skipping one) all give the oracle's bits, with and without codes, distance and interval bounds."""
+    B, CO, CI = 256, 1024, 2048
+    x, w = _data("small_w" if kind == "mixed" else kind, B, CO, CI, 1, seed=31)
+    if kind == "mixed":
+        r = np.random.RandomState(32)
+        x *= 0.05
+        rows = np.arange(0, B, 4)
+        x[rows] = (r.randn(len(rows), CI, 1) * (r.rand(len(rows), CI, 1) < 0.3) * 4).astype(np.float32)
+    eo, ep = O.inf_dist_forward(x, w)
+    out, pos = gpu_inf_forward(x, w)
+    assert np.array_equal(out, eo) and np.array_equal(pos, ep), kind
+    out2, _ = gpu_inf_forward(x, w, with_pos=False)
+    assert np.array_equal(out2, eo), "without codes " + kind
+    xl, xu = _boxes(kind, x, np.random.RandomState(6))
+    expect = O.bound_inf_dist_forward(xl, xu, w)
+    for with_pos in (True, False):
+        got = gpu_bound_forward(xl, xu, w, with_pos=with_pos)
+        for e, v in zip(expect, got):
+            assert v is None or np.array_equal(e, v), "interval bounds " + kind
