@@ -580,6 +580,8 @@ static int launch_row_scaled(FwdParams P, float* scratch, hipStream_t st) {
 
 template <int IP>
 static int launch_sum(const FwdParams& P, hipStream_t st) {
+    if constexpr (IP == 8)  // (with the eight-waves-per-SIMD configurations as candidates 7 and 8, for measurements)
+        return launch_fwd<OpSum<IP>, CfgWide4, CfgBig, CfgSmall, CfgWide, CfgLow32, CfgLow16, CfgWide4H, CfgOcc8, CfgOcc8W>(P, st);
     return launch_fwd<OpSum<IP>, CfgWide4, CfgBig, CfgSmall, CfgWide, CfgLow32, CfgLow16, CfgWide4H>(P, st);
 }
 

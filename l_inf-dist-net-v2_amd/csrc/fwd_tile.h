@@ -74,7 +74,7 @@ struct op_tile_bound : std::false_type {};
 template <class Op>
 struct op_tile_bound<Op, std::enable_if_t<Op::TILE_BOUND>> : std::true_type {};
 
-template <int TM_, int TN_, int WM_, int WN_, int KS_, int KT_ = 32>
+template <int TM_, int TN_, int WM_, int WN_, int KS_, int KT_ = 32, int WAVES_ = 0>
 struct TileCfg {
     static constexpr int TM = TM_, TN = TN_, WM = WM_, WN = WN_, KS = KS_;
     static constexpr int BM = TM * 8 * WM, BN = TN * 8 * WN;
@@ -83,6 +83,10 @@ struct TileCfg {
     static constexpr int KT = KT_;               // k per group per stage == arg-max tile granularity
     static constexpr int KTOT = KT * KS;
     static constexpr int LDM = round_up(BM, 64), LDN = round_up(BN, 64);
+    // waves per SIMD the register allocation must leave room for: four for the 1024-thread workgroups (one per
+    // compute unit), two for the smaller ones, unless the configuration asks for more (two 1024-thread workgroups
+    // per compute unit: eight)
+    static constexpr int WAVES = WAVES_ > 0 ? WAVES_ : (NT >= 1024 ? 4 : 2);
 };
 
 // column of micro-tile slot j for lane index t (0..7) inside a wave-tile that is 8*T wide:
@@ -124,7 +128,7 @@ __device__ __forceinline__ float4 load4_guarded(const float* __restrict__ src, i
 // (a register count just above 256 would halve the occupancy and cost far more than the few spills it avoids).
 // LAYOUT: 0 = [B, C] rows (HW == 1), 1 = [B, C, HW] with positions contiguous, 2 = images with implicit patches
 template <class Op, class Cfg, int LAYOUT>
-__global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::NT >= 1024 ? 4 : 2)))
+__global__ __launch_bounds__(Cfg::NT) __attribute__((amdgpu_waves_per_eu(Cfg::WAVES)))
 void fwd_tile_kernel(const FwdParams P) {
     constexpr int TM = Cfg::TM, TN = Cfg::TN, WN = Cfg::WN, WM = Cfg::WM, BM = Cfg::BM, BN = Cfg::BN;
     constexpr int KT = Cfg::KT, KS = Cfg::KS, KTOT = Cfg::KTOT, NT = Cfg::NT, NTG = Cfg::NTG;
@@ -589,6 +593,10 @@ using CfgLow16 = TileCfg<2, 8, 1, 4, 1>;  // 16 x 256, 256 threads
 // 33 to 64 rows: the 1024-thread tile at half height (64 x 80): four waves per SIMD from one workgroup per compute
 // unit, where the 256-thread 64 x 64 tiles leave the SIMDs with two (p = 8 at 64 x 5120 x 5120: 0.176 -> 0.160 ms)
 using CfgWide4H = TileCfg<4, 5, 2, 2, 4, 16>;
+// the same 64 x 80 tile on 8 k per wave group and stage (48 KB of LDS) within 64 registers: two 1024-thread workgroups
+// per compute unit, eight waves per SIMD (measurement aid: only ever chosen through NORM_DIST_TILE_CFG)
+using CfgOcc8 = TileCfg<4, 5, 2, 2, 4, 8, 8>;
+using CfgOcc8W = TileCfg<4, 5, 4, 2, 2, 16, 8>;  // 128 x 80, 16 k per wave group and stage (64 KB of LDS), likewise
 
 // Second step of a split k range: merges the partial accumulators of one output in split order, finalises, stores.
 template <class Op>
@@ -703,7 +711,7 @@ double tile_cost(const Geom& s, int cus, double part_cost) {
     const double split = Cfg::NT > 256 && ks > 1 ? 1.01 + part_cost * ks : 1.0;  // as in tile_ksplit
     const double few_waves = Cfg::NT <= 256 ? 1.1 : 1.0;
     // measured: at equal padded area the half-height 1024-thread tile is 9 % slower than the full one
-    const double half = std::is_same<Cfg, CfgWide4H>::value ? 1.08 : 1.0;
+    const double half = std::is_same<Cfg, CfgWide4H>::value ? 1.08 : (std::is_same<Cfg, CfgOcc8>::value || std::is_same<Cfg, CfgOcc8W>::value ? 1e3 : 1.0);
     return (double)per_cu * Cfg::BM * Cfg::BN * lds * alone * few_waves * half * split / ks;
 }
 
