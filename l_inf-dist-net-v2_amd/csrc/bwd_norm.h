@@ -18,6 +18,8 @@
 // equal, contiguous share of the units (order: group, slab, row chunk, co chunk), so that grad_x accumulators stay
 // in registers while consecutive units share their rows; they are added to global memory when the rows change.
 #pragma once
+#include <type_traits>
+
 #include "ndist_common.h"
 
 namespace ndist {
@@ -65,6 +67,11 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 // here, which is what the constant address space promises.
 __device__ __forceinline__ f16v load_factors(const float* p) {
     typedef const f16v __attribute__((address_space(4))) * cptr;
+    return *reinterpret_cast<cptr>(reinterpret_cast<uintptr_t>(p));
+}
+typedef float f8v __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ f8v load_factors8(const float* p) {
+    typedef const f8v __attribute__((address_space(4))) * cptr;
     return *reinterpret_cast<cptr>(reinterpret_cast<uintptr_t>(p));
 }
 constexpr int kBwdRowBatch = 16;  // rows whose factors are fetched by one 16-dword scalar load
@@ -572,15 +579,24 @@ __global__ __launch_bounds__(64 * NW, 4) void bwd_fused_kernel(const float* __re
 // registers (complete for this row chunk).  The grad_x partials of the 16 waves are summed through LDS at the end and
 // leave with one global atomic add per element and workgroup (adding them wave by wave would pile a hundred
 // same-address atomics on every element).  The work is bound by streaming w and grad_w.
+// Rows per chunk: 32, or 16 / 8 for batches that small (the arithmetic of the padded rows is the kernel's time there:
+// one to eight rows at 5120 x 5120 took what 32 do).
 constexpr int kBwdSmallRows = 32, kBwdSmallWaves = 16, kBwdSmallMaxM = 32;
+inline int bwd_small_rows(int M) { return M <= 8 ? 8 : (M <= 16 ? 16 : kBwdSmallRows); }
 
-template <int IP, bool WITH_W>
+template <int IP, bool WITH_W, int BT>
 __global__ __launch_bounds__(64 * kBwdSmallWaves) void bwd_small_kernel(const float* __restrict__ X,
                                                                         const float* __restrict__ W,
                                                                         const float* __restrict__ AT,
                                                                         float* __restrict__ GX, float* __restrict__ GW,
                                                                         const BwdParams P, int cosplit, int cows) {
-    constexpr int BT = kBwdSmallRows, RB = kBwdRowBatch, NB = BT / RB, RG = 4;
+    constexpr int RB = BT < kBwdRowBatch ? BT : kBwdRowBatch, NB = BT / RB, RG = 4;
+    static_assert(BT == 8 || BT == 16 || BT == 32, "row chunks of 8, 16 or 32");
+    using FV = typename std::conditional<RB == 16, f16v, f8v>::type;  // one scalar load of RB factors
+    auto load_fv = [](const float* p) __attribute__((always_inline)) -> FV {
+        if constexpr (RB == 16) return load_factors(p);
+        else return load_factors8(p);
+    };
     const Geom& s = P.s;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -608,9 +624,9 @@ __global__ __launch_bounds__(64 * kBwdSmallWaves) void bwd_small_kernel(const fl
     }
     const float* __restrict__ ap = AT + ((long)(g * s.COg + co_begin) * P.Mpad + r0);
     const float* __restrict__ wp = W + w_off(s, g, co_begin, cic);
-    f16v a_cur = load_factors(ap);
-    f16v g_cur = a_cur;
-    if constexpr (IP == -2 || IP == -5) g_cur = load_factors(ap + P.g_off);
+    FV a_cur = load_fv(ap);
+    FV g_cur = a_cur;
+    if constexpr (IP == -2 || IP == -5) g_cur = load_fv(ap + P.g_off);
     float wnext = *wp;
     for (int co = co_begin; co < co_end; co++) {
         const float wv = wnext;
@@ -633,9 +649,9 @@ __global__ __launch_bounds__(64 * kBwdSmallWaves) void bwd_small_kernel(const fl
             __builtin_amdgcn_sched_barrier(0);
             // next batch: same co, next rows; or the next co (after the last co: a harmless re-read of this one)
             const float* __restrict__ apn = bi + 1 < NB ? ap + RB : (last_co ? ap - (NB - 1) * RB : ap + (P.Mpad - (NB - 1) * RB));
-            const f16v a_nxt = load_factors(apn);
-            f16v g_nxt = a_nxt;
-            if constexpr (IP == -2 || IP == -5) g_nxt = load_factors(apn + P.g_off);
+            const FV a_nxt = load_fv(apn);
+            FV g_nxt = a_nxt;
+            if constexpr (IP == -2 || IP == -5) g_nxt = load_fv(apn + P.g_off);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int q0 = RG; q0 < RB; q0 += RG) group(q0);
@@ -651,14 +667,14 @@ __global__ __launch_bounds__(64 * kBwdSmallWaves) void bwd_small_kernel(const fl
         }
     }
     // ---- grad_x: sum over the waves, 16 rows at a time (16 waves x 16 rows x 64 lanes = 64 KB of LDS)
-    constexpr int HR = 16;
+    constexpr int HR = BT < 16 ? BT : 16;
     __shared__ float red[kBwdSmallWaves * HR * kBwdSlab];
 #pragma unroll
     for (int h = 0; h < BT / HR; h++) {
 #pragma unroll
         for (int i = 0; i < HR; i++) red[(wave * HR + i) * kBwdSlab + lane] = gxa[h * HR + i];
         __syncthreads();
-        {
+        if (wave < HR) {
             // thread -> (row = wave index, lane): one cell per thread
             float v = 0.f;
 #pragma unroll
@@ -715,8 +731,19 @@ int launch_bwd_ip_impl(const BwdPtrs& a, const BwdParams& P, int cfg, int grid, 
         }
         const int cows = ceil_div(P.s.COg, cosplit * kBwdSmallWaves);
         const dim3 g3((unsigned)(wgs * cosplit)), b3(64 * kBwdSmallWaves);
-        if (a.gw != nullptr) hipLaunchKernelGGL((bwd_small_kernel<IP, true>), g3, b3, 0, st, a.x, a.w, a.aT, a.gx, a.gw, P, cosplit, cows);
-        else hipLaunchKernelGGL((bwd_small_kernel<IP, false>), g3, b3, 0, st, a.x, a.w, a.aT, a.gx, a.gw, P, cosplit, cows);
+        const int bt = P.Mpad / P.nrc;  // rows per chunk, as the caller laid the factors out (bwd_small_rows)
+#define NDIST_BWD_SMALL(WITH_W, BT_) \
+    hipLaunchKernelGGL((bwd_small_kernel<IP, WITH_W, BT_>), g3, b3, 0, st, a.x, a.w, a.aT, a.gx, a.gw, P, cosplit, cows)
+        if (a.gw != nullptr) {
+            if (bt == 8) NDIST_BWD_SMALL(true, 8);
+            else if (bt == 16) NDIST_BWD_SMALL(true, 16);
+            else NDIST_BWD_SMALL(true, 32);
+        } else {
+            if (bt == 8) NDIST_BWD_SMALL(false, 8);
+            else if (bt == 16) NDIST_BWD_SMALL(false, 16);
+            else NDIST_BWD_SMALL(false, 32);
+        }
+#undef NDIST_BWD_SMALL
         return hip_failed(hipGetLastError()) ? 4 : 0;
     }
     if (a.gw != nullptr) {

@@ -305,7 +305,7 @@ static BwdPlan plan_backward(const Geom& s, float p) {
         }
         if (s.M <= 64) pl.cfg = 4;  // one 64-row chunk (0.33 ms at 5120 x 5120 against 0.51 for a 128-row chunk)
     }
-    pl.rows_per_wg = small ? kBwdSmallRows : kBwdCfgRows[pl.cfg] * kBwdCfgWaves[pl.cfg];
+    pl.rows_per_wg = small ? bwd_small_rows(s.M) : kBwdCfgRows[pl.cfg] * kBwdCfgWaves[pl.cfg];
     return pl;
 }
 
