@@ -111,7 +111,10 @@ def other_workloads(torch, _C, xd, wd, gd):
         for _ in range(n):
             fn()
         torch.cuda.synchronize()
-        return round((time.perf_counter() - t0) * 1e3 / n, 3)
+        ms = (time.perf_counter() - t0) * 1e3 / n
+        if ms < 1.5 and n < 20:  # short calls: five repetitions are within reach of one slow launch
+            return tm(fn, 20)
+        return round(ms, 3)
 
     res = {}
     dev = xd.device

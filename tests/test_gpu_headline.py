@@ -426,3 +426,52 @@ def test_config4_mlp_step_full_size():
     res = np.maximum(m64, 0.0)
     loss64 = 0.75 * res.max(axis=1).mean() + 0.25 * res.mean()
     assert abs(loss.item() - loss64) <= 1e-5 * max(1.0, abs(loss64))
+
+
+def test_config4_mlp_step_full_size_at_p_inf():
+    # The same stack at p = inf, the exponent the reference's schedule ends on and the one certification uses:
+    # every layer's operator call recorded, its forward compared with the oracle over EVERY output (bit-exact
+    # values; the codes through the gradients they route), its backward with the oracle's scatter from the
+    # oracle's own codes.  The layers are identity-initialised, so the library's default path selects the hot
+    # k-tiles by the rows of w.
+    import sys
+    from ell_inf_models import MLPModel, hinge
+    torch.manual_seed(2021)
+    model = MLPModel(depth=6, width=5120, input_dim=(3, 32, 32), identity_val=10.0).cuda()
+    for m in model.modules():
+        if hasattr(m, "p"):
+            m.p = float("inf")
+    x = torch.rand(512, 3, 32, 32, device="cuda")
+    t = torch.randint(0, 10, (512,), device="cuda")
+    eps = 8 / 255 / 0.2009
+    mod = sys.modules["core.modules.norm_dist"]
+    orig = mod.norm_dist
+    calls = []
+
+    def recording(inp, w, p, groups=1, tag=None):
+        inp = inp.detach().requires_grad_(True) if not inp.requires_grad else inp
+        out = orig(inp, w, p, groups, tag=tag)
+        rec = {"x": inp, "w": w, "out": out}
+        inp.register_hook(lambda gr, rec=rec: rec.__setitem__("gx", gr.detach().clone()))
+        out.register_hook(lambda gr, rec=rec: rec.__setitem__("g", gr.detach().clone()))
+        calls.append(rec)
+        return out
+
+    mod.norm_dist = recording
+    try:
+        logits, margin = model(x, targets=t, eps=eps)
+        loss = hinge()(logits, margin, t)
+        loss.backward()
+    finally:
+        mod.norm_dist = orig
+    torch.cuda.synchronize()
+    assert [tuple(c["w"].shape) for c in calls] == [(5120, 3072)] + [(5120, 5120)] * 4 + [(10, 5120)]
+    for li, c in enumerate(calls):
+        xn, wn = c["x"].detach().cpu().numpy(), c["w"].detach().cpu().numpy()
+        eo, ep = O.inf_dist_forward(xn, wn)
+        np.testing.assert_array_equal(c["out"].detach().cpu().numpy(), eo, err_msg="layer %d forward" % li)
+        gn = c["g"].cpu().numpy()
+        ex, ew = O.inf_dist_backward(gn, ep, xn.shape[1])
+        assert_close(c["gx"].cpu().numpy(), ex, what="layer %d grad_input" % li)
+        assert_close(c["w"].grad.cpu().numpy(), ew, what="layer %d grad_weight" % li)
+    assert torch.isfinite(loss)
