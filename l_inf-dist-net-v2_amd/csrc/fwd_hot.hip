@@ -84,7 +84,7 @@ __device__ __forceinline__ void hot_group_maxima(const float* __restrict__ seed_
 //   (dec[4] / dec[5] then say which of them, see below).
 // Cost of a side = its hot entries x the length of the other side.  mode: 1 always the cheaper side, 2 / 3 always
 // the x / w side, else the cheaper side if it touches at most 1 / frac of all (row, column, tile) triples.
-constexpr int kPlanRows = 64, kPlanRowsPerWave = kPlanRows / 16;
+constexpr int kPlanRows = 32, kPlanRowsPerWave = kPlanRows / 16;
 // What differs between two plans over the same weights (a layer's distance and its interval bounds in one call): the
 // rows of the first operand with their statistics, and everything the plan writes.
 struct PlanJob {

@@ -473,5 +473,11 @@ def test_config4_mlp_step_full_size_at_p_inf():
         gn = c["g"].cpu().numpy()
         ex, ew = O.inf_dist_backward(gn, ep, xn.shape[1])
         assert_close(c["gx"].cpu().numpy(), ex, what="layer %d grad_input" % li)
-        assert_close(c["w"].grad.cpu().numpy(), ew, what="layer %d grad_weight" % li)
+        # grad_weight: on these layers every batch row of an output names the same planted weight, and behind a mean
+        # shift the grad_output of an output sums to zero over the batch: the exact gradient is (nearly) zero
+        # everywhere, a sum of 512 terms that cancel.  The error is therefore measured against the size of what is
+        # summed, not against the (vanishing) result.
+        scale = float(np.abs(gn).sum(axis=(0, 2)).max())
+        err = float(np.abs(c["w"].grad.cpu().numpy().astype(np.float64) - ew).max())
+        assert err <= 1e-5 * scale, "layer %d grad_weight: error %.3e against terms summing to %.3e" % (li, err, scale)
     assert torch.isfinite(loss)
