@@ -209,3 +209,21 @@ def test_large_p_probe_in_the_conv_layout():
     _, ew = O.norm_dist_backward(g[:, :4], x, w[:4], out[:, :4], p)
     _, tol = backward_tolerances(g[:, :4], x, w[:4], out[:, :4], p, 1, None, ew)
     assert_close(gw[:4], ew, tol=tol, what="grad_weight")
+
+
+@pytest.mark.parametrize("p", [1.0, 1.5, 2.0, 3.0, 5.0, 8.0, 9.0, 13.7, 100.0])
+@pytest.mark.parametrize("B", [1, 3, 8, 9, 16, 17, 32])
+def test_backward_row_chunks_of_small_batches(B, p):
+    # the small-batch backward works on chunks of 8, 16 or 32 rows (reference: the same kernels for every batch size,
+    # core/cuda/norm_dist_cuda.cu:590-623): every exponent family at batch sizes on and next to the chunk borders,
+    # both entry points, two groups, ragged co and ci
+    CO, CI, G = 52, 330, 2
+    x, w, g = make_inputs(1200 + B, B, CO, CI, G, 1)
+    out = gpu_norm_forward(x, w, p, G)
+    ex, ew = O.norm_dist_backward(g, x, w, out, p, G)
+    gx, gw = gpu_norm_backward(g, x, w, out, p, G)
+    tol_x, tol_w = backward_tolerances(g, x, w, out, p, G, ex, ew)
+    assert_close(gx, ex, tol=tol_x, what="grad_input B=%d p=%g" % (B, p))
+    assert_close(gw, ew, tol=tol_w, what="grad_weight B=%d p=%g" % (B, p))
+    gx2, _ = gpu_norm_backward(g, x, w, out, p, G, with_weight=False)
+    assert_close(gx2, ex, tol=tol_x, what="input-only entry point B=%d p=%g" % (B, p))
