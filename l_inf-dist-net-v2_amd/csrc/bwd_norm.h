@@ -40,6 +40,8 @@ struct BwdParams {
     Geom s;
     int Mpad;         // rows padded to a multiple of NW*BT; padding carries g = 0
     int nslab, ncc, nrc;
+    int gw_add;       // grad_weight is added to (atomics into a gradient zeroed beforehand): several row chunks, or a
+                      // caller that accumulates over several launches; 0: stored
     long total;       // G * nslab * nrc * ncc units
     float q;          // p - 1
     // term-skipping variant (IP == -3): terms below 2^-40 * max|grad_output| are dropped; gmax points at that maximum
@@ -562,7 +564,7 @@ __global__ __launch_bounds__(64 * NW, 4) void bwd_fused_kernel(const float* __re
                 const int cl = idx >> 6, l = idx & 63;
                 if (cur.ci0 + l < s.CIg) {
                     float* dst = GW + w_off(s, cur.g, cur.co0 + cl, cur.ci0 + l);
-                    if (P.nrc == 1) *dst = -v;
+                    if (!P.gw_add) *dst = -v;
                     else atomicAdd(dst, -v);
                 }
             }
@@ -662,7 +664,7 @@ __global__ __launch_bounds__(64 * kBwdSmallWaves) void bwd_small_kernel(const fl
         if (WITH_W && ci_ok) {
             const float v = -((gwp[0] + gwp[1]) + (gwp[2] + gwp[3]));
             float* dst = GW + w_off(s, g, co, ci);
-            if (P.nrc == 1) *dst = v;
+            if (!P.gw_add) *dst = v;
             else atomicAdd(dst, v);
         }
     }

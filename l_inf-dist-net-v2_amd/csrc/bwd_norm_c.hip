@@ -304,6 +304,9 @@ static BwdPlan plan_backward(const Geom& s, float p) {
             if (c == 0 || cost < best) { best = cost; pl.cfg = c; }
         }
         if (s.M <= 64) pl.cfg = 4;  // one 64-row chunk (0.33 ms at 5120 x 5120 against 0.51 for a 128-row chunk)
+        // tuning aid: NORM_DIST_BWD_CFG=0 / 1 / 2 forces the 16- / 8- / 4-wave workgroups
+        static const char* force = getenv("NORM_DIST_BWD_CFG");
+        if (force != nullptr && force[0] >= '0' && force[0] <= '2') pl.cfg = force[0] - '0';
     }
     pl.rows_per_wg = small ? bwd_small_rows(s.M) : kBwdCfgRows[pl.cfg] * kBwdCfgWaves[pl.cfg];
     return pl;
@@ -316,7 +319,7 @@ size_t norm_backward_scratch_bytes(const Geom& s, float p) {
 }
 
 int launch_norm_backward(const float* gout, const float* x, const float* w, const float* out, const Geom& s, float* gx,
-                         float* gw, float p, hipStream_t st, const UnfoldGeom* cv) {
+                         float* gw, float p, hipStream_t st, const UnfoldGeom* cv, bool gw_accumulate) {
     const float q = p - 1.0f;
     const BwdPlan pl = plan_backward(s, p);
     const int ip = pl.ip, cfg = pl.cfg;
@@ -331,6 +334,7 @@ int launch_norm_backward(const float* gout, const float* x, const float* w, cons
     P.ncc = ceil_div(s.COg, kBwdCoUnit);
     P.total = (long)s.G * P.nslab * P.nrc * P.ncc;
     P.q = q;
+    P.gw_add = P.nrc > 1 || gw_accumulate ? 1 : 0;
 
     const size_t tbytes = (size_t)s.COg * s.G * P.Mpad * sizeof(float);
     float* aT = nullptr;
@@ -415,7 +419,7 @@ int launch_norm_backward(const float* gout, const float* x, const float* w, cons
     }
     P.part = part;
     if (!rc && part == nullptr) rc = fill_zero(gx_k, nx, st);
-    if (!rc && gw != nullptr && P.nrc > 1) rc = fill_zero(gw, (long)s.COg * s.G * s.CIg, st);
+    if (!rc && gw != nullptr && P.nrc > 1 && !gw_accumulate) rc = fill_zero(gw, (long)s.COg * s.G * s.CIg, st);
     if (!rc) {
         // Persistent workgroups take equal shares of the units, so all of them should be resident at once: two 8-wave
         // workgroups fit a compute unit (72 KB of LDS each), four 4-wave ones (40 KB each, exactly the 160 KB) and six

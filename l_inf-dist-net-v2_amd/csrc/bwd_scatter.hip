@@ -480,6 +480,10 @@ static int scatter_backward(const float* g1, const float* g2, const int32_t* p1,
             // short segments, and four workgroups of 2 x 20 KB per compute unit overlap their fill, scatter and
             // store phases better than two of 4 x 20 KB (31.7 against 36.5 us at 512 x 5120 x 5120)
             R = R > 2 ? 2 : R;
+            {   // tuning aid: NORM_DIST_GW_ROWS=<n> rows of grad_weight per workgroup
+                static const char* force = getenv("NORM_DIST_GW_ROWS");
+                if (force != nullptr && atoi(force) >= 1) R = atoi(force) < R ? atoi(force) : R;
+            }
             hipLaunchKernelGGL(scatter_gw_rows_kernel<BOUND>, dim3(ceil_div(s.COg, R), s.G), dim3(256),
                                (size_t)R * s.CIg * sizeof(float), st, g1, g2, p1, p2, gw, s, R);
             if (hip_failed(hipGetLastError())) return 4;

@@ -3,6 +3,7 @@
 // what the reference's binding layer enforces (core/cuda/norm_dist.cpp:8-12) as far as raw pointers allow.
 #include "../../include/norm_dist_hip.h"
 
+#include <algorithm>
 #include <atomic>
 #include <cmath>
 #include <mutex>
@@ -503,8 +504,38 @@ static int conv_norm_backward(const float* grad_output, const float* input, cons
     if (int rc = make_conv_geom(B, C, H, W, CO, G, kernel_h, kernel_w, dilation_h, dilation_w, padding_h, padding_w,
                                 stride_h, stride_w, &u, &s))
         return rc;
-    return launch_norm_backward(grad_output, input, weight, output, s, grad_input, grad_weight, p, (hipStream_t)stream,
-                                &u);
+    // The backward's kernel reads the patches as rows and writes gradient rows: two buffers of the unfolded size
+    // (B x C kh kw x OH OW floats each, 604 MB at 128 x 128 x 32 x 32 with 3 x 3 windows).  Batches whose buffers
+    // would exceed 256 MiB each are processed in parts of whole samples, grad_weight accumulating
+    // over the parts: the scratch stays bounded whatever the batch, at no cost in time (the parts are long enough to
+    // fill the device and grad_weight is added with atomics from the second row chunk on anyway).
+    size_t budget = 256u << 20;
+    if (const char* mb = getenv("NORM_DIST_CONV_PART_MB")) {  // tuning / test aid: budget per buffer in MiB
+        if (atol(mb) > 0) budget = (size_t)atol(mb) << 20;
+    }
+    const size_t per_sample = (size_t)s.CIg * s.G * s.HW * sizeof(float);
+    int part = (int)std::max<size_t>(1, budget / std::max<size_t>(1, per_sample));
+    part = ceil_div(B, ceil_div(B, part));  // parts of equal size
+    if (B <= part)
+        return launch_norm_backward(grad_output, input, weight, output, s, grad_input, grad_weight, p,
+                                    (hipStream_t)stream, &u);
+    if (grad_weight != nullptr) {
+        if (int rc = fill_zero(grad_weight, (long)s.COg * s.G * s.CIg, (hipStream_t)stream)) return rc;
+    }
+    const long out_stride = (long)CO * s.HW, img_stride = (long)C * H * W;
+    for (int b0 = 0; b0 < B; b0 += part) {
+        const int nb = std::min(part, B - b0);
+        UnfoldGeom up;
+        Geom sp;
+        if (int rc = make_conv_geom(nb, C, H, W, CO, G, kernel_h, kernel_w, dilation_h, dilation_w, padding_h, padding_w,
+                                    stride_h, stride_w, &up, &sp))
+            return rc;
+        if (int rc = launch_norm_backward(grad_output + b0 * out_stride, input + b0 * img_stride, weight,
+                                          output + b0 * out_stride, sp, grad_input + b0 * img_stride, grad_weight, p,
+                                          (hipStream_t)stream, &up, grad_weight != nullptr))
+            return rc;
+    }
+    return NDIST_OK;
 }
 
 int ndist_conv_norm_dist_backward_input(const float* grad_output, const float* input, const float* weight,

@@ -306,8 +306,11 @@ int launch_norm_forward_conv(const float* x, const float* w, const Geom& s, floa
                              const UnfoldGeom& cv);
 // With a patch geometry x and gx are images [B, C, H, W] and s describes the unfolded problem: the patches go
 // straight into the row layout the kernel reads and the gradient rows are folded back into the image.
+// gw_accumulate: grad_weight was zeroed by the caller and is added to (several launches over parts of a batch).
 int launch_norm_backward(const float* gout, const float* x, const float* w, const float* out, const Geom& s,
-                         float* gx, float* gw, float p, hipStream_t st, const UnfoldGeom* cv = nullptr);
+                         float* gx, float* gw, float p, hipStream_t st, const UnfoldGeom* cv = nullptr,
+                         bool gw_accumulate = false);
+int fill_zero(float* p, long n, hipStream_t st);
 // bytes of scratch launch_norm_backward cannot do without (the factor array); everything else it asks for is optional
 size_t norm_backward_scratch_bytes(const Geom& s, float p);
 // With a patch geometry the input gradients are images [B, C, H, W] (the adjoint of the patch extraction is applied
