@@ -499,6 +499,16 @@ __global__ __launch_bounds__(64 * NW, 4) void bwd_fused_kernel(const float* __re
 #pragma unroll
                 for (int k = 0; k < 4; k++) avq[k] = load_av(ap_next_unit, k, nn);
             }
+        } else if (xr0 >= s.M) {
+            // every row of this wave is padding of the last row chunk (x and the factors are zero there): nothing to
+            // add; its grad_weight slots read as zero, and the factor requests go on with the next unit's first batch
+            if (WITH_W) {
+                for (int c = 0; c < cur.co1 - cur.co0; c++) mine[c * kBwdSlab] = 0.f;
+            }
+            ap = ap_next_unit;
+            a_cur = load_factors(ap);
+            g_cur = a_cur;
+            if constexpr (IP == -2 || IP == -5) g_cur = load_factors(ap + P.g_off);
         } else
         for (int co = cur.co0; co < cur.co1; co++) {
             const float wv = wnext;
