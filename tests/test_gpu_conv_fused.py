@@ -249,34 +249,35 @@ def test_conv_norm_dist_layer_matches_the_unfolded_path():
     assert_close(gw.cpu().numpy(), layer.weight.grad.cpu().numpy(), what="layer grad_weight")
 
 
+@pytest.mark.parametrize("G,stride", [(1, 1), (2, 2)])
 @pytest.mark.parametrize("p", [3.0, 13.7])
-def test_conv_norm_dist_backward_in_parts_of_the_batch(p, monkeypatch):
+def test_conv_norm_dist_backward_in_parts_of_the_batch(p, G, stride, monkeypatch):
     """Large batches run the finite-p backward on images in parts of whole samples, so that the two patch-sized
     scratch buffers stay bounded, grad_weight accumulating over the parts.  With the budget forced down to 1 MiB per
-    buffer (590 KB of patches per sample here) a 7-sample batch takes seven parts: same gradients as in one piece,
-    within 1e-5 of the oracle."""
+    buffer (590 KB of patches per sample at stride 1, 147 KB at stride 2) a 9-sample batch takes nine parts, or two
+    of five and four samples: same gradients as in one piece, within 1e-5 of the oracle; also with groups."""
     from core import _C
     from util import backward_tolerances
-    B, C, H, W, CO, k = 7, 16, 32, 32, 10, 3
+    B, C, H, W, CO, k = 9, 16, 32, 32, 10, 3
     gen = torch.Generator().manual_seed(77)
     x = torch.randn(B, C, H, W, generator=gen)
-    w = torch.randn(CO, C * k * k, generator=gen) / (C * k * k) ** 0.5
-    patches = F.unfold(x, k, 1, 1, 1)
+    w = torch.randn(CO, C // G * k * k, generator=gen) / (C * k * k) ** 0.5
+    patches = F.unfold(x, k, 1, 1, stride)
     xd, wd = x.cuda(), w.cuda()
     out = torch.empty(B, CO, patches.size(2), device="cuda")
-    _C.conv_norm_dist_forward(xd, wd, out, 1, p, k, 1, 1, 1)
+    _C.conv_norm_dist_forward(xd, wd, out, G, p, k, 1, 1, stride)
     g = torch.randn(out.shape, generator=gen)
-    ex, ew = O.norm_dist_backward(g.numpy(), patches.numpy(), w.numpy(), out.cpu().numpy(), p, 1)
-    ex_img = F.fold(torch.from_numpy(ex), (H, W), k, 1, 1, 1).numpy()
-    tol_x, tol_w = backward_tolerances(g.numpy(), patches.numpy(), w.numpy(), out.cpu().numpy(), p, 1, ex, ew)
+    ex, ew = O.norm_dist_backward(g.numpy(), patches.numpy(), w.numpy(), out.cpu().numpy(), p, G)
+    ex_img = F.fold(torch.from_numpy(ex), (H, W), k, 1, 1, stride).numpy()
+    tol_x, tol_w = backward_tolerances(g.numpy(), patches.numpy(), w.numpy(), out.cpu().numpy(), p, G, ex, ew)
     whole = [torch.full_like(xd, float("nan")), torch.full_like(wd, float("nan"))]
-    _C.conv_norm_dist_backward_input_weight(g.cuda(), xd, wd, out, whole[0], whole[1], 1, p, k, 1, 1, 1)
+    _C.conv_norm_dist_backward_input_weight(g.cuda(), xd, wd, out, whole[0], whole[1], G, p, k, 1, 1, stride)
     monkeypatch.setenv("NORM_DIST_CONV_PART_MB", "1")
     parts = [torch.full_like(xd, float("nan")), torch.full_like(wd, float("nan"))]
-    _C.conv_norm_dist_backward_input_weight(g.cuda(), xd, wd, out, parts[0], parts[1], 1, p, k, 1, 1, 1)
+    _C.conv_norm_dist_backward_input_weight(g.cuda(), xd, wd, out, parts[0], parts[1], G, p, k, 1, 1, stride)
     for got in (whole, parts):
         assert_close(got[0].cpu().numpy(), ex_img, tol=tol_x, what="grad_input p=%g" % p)
         assert_close(got[1].cpu().numpy(), ew, tol=tol_w, what="grad_weight p=%g" % p)
     only_x = torch.full_like(xd, float("nan"))
-    _C.conv_norm_dist_backward_input(g.cuda(), xd, wd, out, only_x, 1, p, k, 1, 1, 1)
+    _C.conv_norm_dist_backward_input(g.cuda(), xd, wd, out, only_x, G, p, k, 1, 1, stride)
     assert_close(only_x.cpu().numpy(), ex_img, tol=tol_x, what="input-only entry point in parts p=%g" % p)
