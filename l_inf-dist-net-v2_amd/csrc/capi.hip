@@ -507,8 +507,9 @@ static int conv_norm_backward(const float* grad_output, const float* input, cons
     // The backward's kernel reads the patches as rows and writes gradient rows: two buffers of the unfolded size
     // (B x C kh kw x OH OW floats each, 604 MB at 128 x 128 x 32 x 32 with 3 x 3 windows).  Batches whose buffers
     // would exceed 256 MiB each are processed in parts of whole samples, grad_weight accumulating
-    // over the parts: the scratch stays bounded whatever the batch, at no cost in time (the parts are long enough to
-    // fill the device and grad_weight is added with atomics from the second row chunk on anyway).
+    // over the parts: the scratch stays bounded whatever the batch, at a small cost in time (the parts are long enough
+    // to fill the device and grad_weight is added with atomics from the second row chunk on anyway: three parts of
+    // 43 samples at that shape take 4 % longer than one piece).
     size_t budget = 256u << 20;
     if (const char* mb = getenv("NORM_DIST_CONV_PART_MB")) {  // tuning / test aid: budget per buffer in MiB
         if (atol(mb) > 0) budget = (size_t)atol(mb) << 20;
