@@ -21,6 +21,7 @@ template <bool TRACK, bool BOUNDED = false>
 struct OpBound {
     static constexpr int NX = 2, PHASES = 1, NOF = 2, NOI = TRACK ? 2 : 0;
     static constexpr bool PREFETCH = false;  // two x arrays: the operand set is already large
+    static constexpr bool PREFETCH_SMALL = true;
     static constexpr bool TILE_BOUND = BOUNDED;
     static constexpr float COST = TRACK ? 18.f : 15.f;  // issue cycles per pair and wave (launcher's cost model)
     struct AccPlain { float lo, hi; };

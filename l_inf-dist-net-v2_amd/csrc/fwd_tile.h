@@ -74,6 +74,13 @@ struct op_tile_bound : std::false_type {};
 template <class Op>
 struct op_tile_bound<Op, std::enable_if_t<Op::TILE_BOUND>> : std::true_type {};
 
+// policies whose 256-thread configurations (two waves per SIMD, 256 registers) have room for a second operand set
+// although their 1024-thread ones do not: `static constexpr bool PREFETCH_SMALL = true`
+template <class Op, class = void>
+struct op_prefetch_small : std::false_type {};
+template <class Op>
+struct op_prefetch_small<Op, std::enable_if_t<Op::PREFETCH_SMALL>> : std::true_type {};
+
 template <int TM_, int TN_, int WM_, int WN_, int KS_, int KT_ = 32, int WAVES_ = 0>
 struct TileCfg {
     static constexpr int TM = TM_, TN = TN_, WM = WM_, WN = WN_, KS = KS_;
@@ -402,15 +409,20 @@ void fwd_tile_kernel(const FwdParams P) {
                                           NX == 2 ? c1[slot][i] : 0.f, b1[slot]);
             };
             static_assert(KT % 4 == 0, "two steps of two k per iteration");
-            if constexpr (Op::PREFETCH && NT <= 512) {
+            if constexpr ((Op::PREFETCH && NT <= 512) || (op_prefetch_small<Op>::value && NT <= 256)) {
+                // (the last iteration is peeled: a read under a condition at the end of the loop body makes the
+                // compiler carry both operand sets through copies, one v_mov per register and iteration)
                 read_step(0, 0);
 #pragma unroll 1
-                for (int kk = 0; kk < KT; kk += 4) {
+                for (int kk = 0; kk < KT - 4; kk += 4) {
                     read_step(kk + 2, 1);
                     compute_step(0);
-                    if (kk + 4 < KT) read_step(kk + 4, 0);
+                    read_step(kk + 4, 0);
                     compute_step(1);
                 }
+                read_step(KT - 2, 1);
+                compute_step(0);
+                compute_step(1);
             } else {  // register-hungry accumulators: no room for a second operand set
 #pragma unroll 2
                 for (int kk = 0; kk < KT; kk += 2) {
