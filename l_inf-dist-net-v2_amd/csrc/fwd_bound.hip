@@ -22,6 +22,7 @@ struct OpBound {
     static constexpr int NX = 2, PHASES = 1, NOF = 2, NOI = TRACK ? 2 : 0;
     static constexpr bool PREFETCH = false;  // two x arrays: the operand set is already large
     static constexpr bool PREFETCH_SMALL = true;
+    static constexpr bool HEAVY = true;
     static constexpr bool TILE_BOUND = BOUNDED;
     static constexpr float COST = TRACK ? 18.f : 15.f;  // issue cycles per pair and wave (launcher's cost model)
     struct AccPlain { float lo, hi; };
@@ -186,7 +187,7 @@ int launch_bound_forward(const float* xl, const float* xu, const float* w, const
     // large fully-connected problems: hot-tile kernels first, else seeds and k-tile bounds, as in launch_inf_forward
     const bool bounded = cv == nullptr && seeded_forward_applies(s);
     const bool hot = cv == nullptr && hot_forward_applies(s) && (bounded || hot_alone_applies(s));
-    if (!bounded && !hot && pl == nullptr) return launch_fwd_conv<OpBound<false>, CfgBoundN, CfgMid, CfgSmall>(P, st);
+    if (!bounded && !hot && pl == nullptr) return launch_fwd_conv<OpBound<false>, CfgBoundN, CfgSmall>(P, st);
     KernelTimer timer(st);  // pre-passes + tiled kernel + rescan
     float* scratch = nullptr;
     const int* gate = nullptr;
@@ -239,8 +240,8 @@ int launch_bound_forward(const float* xl, const float* xu, const float* w, const
     }
     if (pl == nullptr) {
         int rc = bounded ? launch_fwd<OpBound<false, true>, CfgBoundT, CfgMid, CfgSmall>(P, st)
-                         : launch_fwd_conv<OpBound<false>, CfgBoundN, CfgMid, CfgSmall>(P, st);
-        if (!rc && two) rc = launch_fwd_conv<OpBound<false>, CfgBoundN, CfgMid, CfgSmall>(Q, st);
+                         : launch_fwd_conv<OpBound<false>, CfgBoundN, CfgSmall>(P, st);
+        if (!rc && two) rc = launch_fwd_conv<OpBound<false>, CfgBoundN, CfgSmall>(Q, st);
         return done(rc);
     }
     int kt = 0;

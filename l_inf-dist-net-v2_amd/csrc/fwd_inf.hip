@@ -25,6 +25,7 @@ struct OpInf {
     static constexpr int NX = 1, PHASES = 1, NOF = 1, NOI = TRACK ? 1 : 0;
     static constexpr bool PREFETCH = !TRACK;
     static constexpr bool PREFETCH_SMALL = true;
+    static constexpr bool HEAVY = TRACK;
     static constexpr bool TILE_BOUND = BOUNDED;
     static constexpr float COST = TRACK ? 6.2f : 5.2f;  // issue cycles per pair and wave (launcher's cost model)
     struct AccPlain { float m; };

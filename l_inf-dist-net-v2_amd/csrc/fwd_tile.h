@@ -713,7 +713,15 @@ double split_part_cost(const Geom& s) {
 // the LDS traffic of the micro-tile shape, divided by the split of the k range.  A 256-thread workgroup alone on its
 // compute unit (one wave per SIMD, nothing to hide latencies behind) runs at little more than half its speed.
 // Measured on top of that: per pair the 256-thread tiles are 7 % to 15 % slower than the 512- and 1024-thread ones.
-template <class Cfg>
+// Policies with several registers of state per output (arg-max bookkeeping, two reductions of the interval bounds):
+// `static constexpr bool HEAVY = true`.  Their 128 x 64 tiles run two waves per SIMD where the 64 x 64 ones run
+// three, and measure 0 - 20 % slower per pair (6 % on the 3 x 3 convolution with 128 channels).
+template <class Op, class = void>
+struct op_heavy : std::false_type {};
+template <class Op>
+struct op_heavy<Op, std::enable_if_t<Op::HEAVY>> : std::true_type {};
+
+template <class Op, class Cfg>
 double tile_cost(const Geom& s, int cus, double part_cost) {
     const int ks = tile_ksplit<Cfg>(s, cus, part_cost);
     const long tiles = (long)ceil_div(s.M, Cfg::BM) * ceil_div(s.COg, Cfg::BN) * s.G * ks;
@@ -724,7 +732,8 @@ double tile_cost(const Geom& s, int cus, double part_cost) {
     const double few_waves = Cfg::NT <= 256 ? 1.1 : 1.0;
     // measured: at equal padded area the half-height 1024-thread tile is 9 % slower than the full one
     const double half = std::is_same<Cfg, CfgWide4H>::value ? 1.08 : (std::is_same<Cfg, CfgOcc8>::value || std::is_same<Cfg, CfgOcc8W>::value ? 1e3 : 1.0);
-    return (double)per_cu * Cfg::BM * Cfg::BN * lds * alone * few_waves * half * split / ks;
+    const double two_waves = op_heavy<Op>::value && std::is_same<Cfg, CfgMid>::value ? 1.08 : 1.0;
+    return (double)per_cu * Cfg::BM * Cfg::BN * lds * alone * few_waves * half * two_waves * split / ks;
 }
 
 }  // namespace ndist
@@ -751,7 +760,7 @@ int launch_fwd_layouts(FwdParams P, hipStream_t st, int* chosen_kt = nullptr) {
               (P.pos2 == nullptr || (uintptr_t)P.pos2 % 16 == 0);
     const int cus = device_info().num_cu;
     const double part_cost = split_part_cost<Op>(s);
-    const double costs[] = {tile_cost<Cfgs>(s, cus, part_cost)...};
+    const double costs[] = {tile_cost<Op, Cfgs>(s, cus, part_cost)...};
     int best = 0;
     for (int i = 1; i < (int)sizeof...(Cfgs); i++)
         if (costs[i] < costs[best]) best = i;
