@@ -236,10 +236,10 @@ int launch_inf_forward(const float* x, const float* w, const Geom& s, float* out
     }
     int kt = 0;
     int rc = bounded ? launch_fwd_layouts<false, OpInf<true, true>, CfgWideT, CfgMid, CfgSmall>(P, st, &kt)
-                     : launch_fwd_layouts<true, OpInf<true>, CfgWideT, CfgMid, CfgSmall>(P, st, &kt);
+                     : launch_fwd_layouts<true, OpInf<true>, CfgWideT, CfgMid, CfgSmall4>(P, st, &kt);
     if (!rc && two) {
         int kt2 = 0;
-        rc = launch_fwd_layouts<true, OpInf<true>, CfgWideT, CfgMid, CfgSmall>(Q, st, &kt2);
+        rc = launch_fwd_layouts<true, OpInf<true>, CfgWideT, CfgMid, CfgSmall4>(Q, st, &kt2);
         if (!rc && kt2 != kt) rc = 2;  // (same candidate list and cost model: cannot differ)
     }
     if (rc) return done(rc);
