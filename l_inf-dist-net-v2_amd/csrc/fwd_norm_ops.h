@@ -126,6 +126,8 @@ template <bool GIVEN_MAX>
 struct OpNormalized {
     static constexpr int NX = 1, PHASES = GIVEN_MAX ? 1 : 2, NOF = 1, NOI = 0;
     static constexpr bool PREFETCH = false;  // three registers per output: no room for a second operand set
+    static constexpr bool PREFETCH_SMALL = true;
+    static constexpr bool HEAVY = true;
     static constexpr float COST = GIVEN_MAX ? 25.8f : 35.9f;
     struct Acc { float m, c, s; };
     __device__ static __forceinline__ void init(Acc& a, const FwdParams& P, int kg, int m, int n, int g) {
