@@ -241,12 +241,25 @@ def _fused_conv_ok(*tensors):
     return all(t.is_cuda and t.dtype == torch.float32 and t.dim() == 4 for t in tensors)
 
 
+def _empty_batch(shape, count, *tensors):
+    """An empty batch.  The reference's kernels are launched over no rows then and leave an empty output, and its
+    backward clears grad_weight before a launch that does nothing (core/cuda/norm_dist_cuda.cu:515-520, 602-604); the
+    C ABI here refuses empty shapes, so the empty outputs are formed on the host, tied to the inputs and the weight
+    so that these receive zero gradients."""
+    tie = sum(t.sum() * 0 for t in tensors)
+    outs = tuple(tensors[0].new_zeros(shape) + tie for _ in range(count))
+    return outs[0] if count == 1 else outs
+
+
 def conv_norm_dist(input, weight, p, kernel_size, dilation=1, padding=0, stride=1, groups=1, tag=None):
     """norm_dist(unfold(input), weight, p, groups) for images [B, C, H, W] (what the reference's NormDistConv
     computes, core/modules/norm_dist.py:93-102).  At p = inf the kernels extract the patches while they load their
     tiles and scatter the gradient straight into the image: neither the unfolded tensor nor its gradient is ever
     written; values and arg-max codes are bit-identical.  Finite p works on the image too: the forward extracts the
     patches on the fly, the backward writes them once as rows for its kernel and folds the gradient rows back."""
+    if input.size(0) == 0:
+        _, (oh, ow) = _C.unfold_geometry(input.shape, kernel_size, dilation, padding, stride)
+        return _empty_batch((0, weight.size(0), oh * ow), 1, input, weight)
     need_grad = torch.is_grad_enabled() and (input.requires_grad or weight.requires_grad)
     if not math.isinf(p) and _fused_conv_ok(input) and weight.is_cuda:
         if p <= 0:
@@ -272,6 +285,9 @@ def conv_norm_dist(input, weight, p, kernel_size, dilation=1, padding=0, stride=
 def conv_bound_inf_dist(x_lower, x_upper, weight, kernel_size, dilation=1, padding=0, stride=1, groups=1, tag=None):
     """bound_inf_dist(unfold(x_lower), unfold(x_upper), weight, groups) for image boxes [B, C, H, W]; fused like
     conv_norm_dist."""
+    if x_lower.size(0) == 0:
+        _, (oh, ow) = _C.unfold_geometry(x_lower.shape, kernel_size, dilation, padding, stride)
+        return _empty_batch((0, weight.size(0), oh * ow), 2, x_lower, x_upper, weight)
     need_grad = torch.is_grad_enabled() and (x_lower.requires_grad or x_upper.requires_grad or weight.requires_grad)
     if need_grad and _fused_conv_ok(x_lower, x_upper):
         return ConvBoundInfDistF.apply(x_lower.contiguous(), x_upper.contiguous(), weight.contiguous(), groups,
@@ -331,6 +347,8 @@ class WeightCache:
 def inf_dist_nograd(x, weight, groups=1, cache=None):
     """The infinity distance without gradients, optionally with the weights' pre-pass taken from `cache`
     (WeightCache)."""
+    if x.size(0) == 0:
+        return _new_output(x, weight)
     buffer = cache.get(weight, groups) if cache is not None else None
     x, weight = x.contiguous(), weight.contiguous()
     y = _new_output(x, weight)
@@ -347,7 +365,7 @@ def inf_dist_with_bounds(x, x_lower, x_upper, weight, groups=1, tag=None, cache=
     operator calls).  Without gradients the two run as one library call that shares the pre-pass over the weights;
     with gradients they are the two autograd operators."""
     tensors = (x, x_lower, x_upper, weight)
-    if (all(t.is_cuda and t.dtype == torch.float32 for t in tensors)
+    if (x.size(0) > 0 and all(t.is_cuda and t.dtype == torch.float32 for t in tensors)
             and not (torch.is_grad_enabled() and any(t.requires_grad for t in tensors))):
         buffer = cache.get(weight, groups) if cache is not None else None
         x, x_lower, x_upper, weight = (t.contiguous() for t in tensors)
@@ -420,6 +438,8 @@ def _grouped(t, groups):
 
 
 def norm_dist(input, weight, p, groups=1, use_custom_cuda_func=True, tag=None):
+    if use_custom_cuda_func and input.size(0) == 0:
+        return _empty_batch((0, weight.size(0), input.size(2)), 1, input, weight)
     if use_custom_cuda_func:
         need_grad = torch.is_grad_enabled() and (input.requires_grad or weight.requires_grad)
         return NormDistF.apply(input, weight, groups, p, need_grad, tag)
@@ -431,6 +451,8 @@ def norm_dist(input, weight, p, groups=1, use_custom_cuda_func=True, tag=None):
 
 
 def bound_inf_dist(x_lower, x_upper, weight, groups=1, use_custom_cuda_func=True, tag=None):
+    if use_custom_cuda_func and x_lower.size(0) == 0:
+        return _empty_batch((0, weight.size(0), x_lower.size(2)), 2, x_lower, x_upper, weight)
     if use_custom_cuda_func:
         need_grad = torch.is_grad_enabled() and (x_lower.requires_grad or x_upper.requires_grad or weight.requires_grad)
         return BoundInfDistF.apply(x_lower, x_upper, weight, groups, need_grad, tag)

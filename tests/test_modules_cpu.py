@@ -115,3 +115,26 @@ def test_bound_sequential_threads_the_triple():
     x = torch.randn(2, 3)
     y, lo, up = seq((x, x - 0.1, x + 0.1))
     assert bool((lo <= y + 1e-6).all()) and bool((y <= up + 1e-6).all()) and bool((lo >= 0).all())
+
+
+@pytest.mark.parametrize("p", [8.0, float("inf")])
+def test_an_empty_batch_gives_empty_outputs_and_zero_gradients(p):
+    """The reference's kernels run over no rows on an empty batch and its backward clears grad_weight before a launch
+    that does nothing (core/cuda/norm_dist_cuda.cu:515-520, 602-604): empty outputs, zero gradients, no error."""
+    from core.norm_dist import conv_norm_dist, conv_bound_inf_dist
+    w = torch.randn(6, 8, requires_grad=True)
+    x = torch.zeros(0, 8, 3, requires_grad=True)
+    y = norm_dist(x, w, p)
+    assert y.shape == (0, 6, 3)
+    y.sum().backward()
+    assert x.grad.shape == x.shape and torch.equal(w.grad, torch.zeros_like(w))
+    lo, up = bound_inf_dist(x.detach(), x.detach(), w)
+    assert lo.shape == up.shape == (0, 6, 3)
+    wc = torch.randn(5, 4 * 9, requires_grad=True)
+    img = torch.zeros(0, 4, 7, 7, requires_grad=True)
+    yc = conv_norm_dist(img, wc, p, 3, 1, 1, 2)
+    assert yc.shape == (0, 5, 16)
+    yc.sum().backward()
+    assert torch.equal(wc.grad, torch.zeros_like(wc)) and img.grad.shape == img.shape
+    cl, cu = conv_bound_inf_dist(img.detach(), img.detach(), wc, 3, 1, 1, 2)
+    assert cl.shape == cu.shape == (0, 5, 16)
