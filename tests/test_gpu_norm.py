@@ -98,6 +98,20 @@ def test_backward_more_shapes(B, CO, CI, p):
     assert_close(gw, ew, what="grad_weight")
 
 
+@pytest.mark.parametrize("p", [1.5, 100.0, 200.0])
+@pytest.mark.parametrize("B,CO,CI", [(65, 40, 200), (130, 50, 130), (300, 33, 70)])
+def test_backward_padded_row_chunks_with_a_second_factor_array(B, CO, CI, p):
+    """Waves whose rows are all padding of the last row chunk skip their units; the variants that read a second factor
+    array (grad_output apart below p = 2, the compensation term from p = 65 on) must keep both request streams going."""
+    x, w, g = make_inputs(900 + B, B, CO, CI)
+    out = O.norm_dist_forward(x, w, p).astype(np.float32)
+    ex, ew = O.norm_dist_backward(g, x, w, out, p)
+    gx, gw = gpu_norm_backward(g, x, w, out, p)
+    tol_x, tol_w = backward_tolerances(g, x, w, out, p, 1, ex, ew)
+    assert_close(gx, ex, tol=tol_x, what="grad_input B=%d p=%g" % (B, p))
+    assert_close(gw, ew, tol=tol_w, what="grad_weight B=%d p=%g" % (B, p))
+
+
 @pytest.mark.parametrize("p", [1.0, 1.5, 8.0, 13.7])
 @pytest.mark.parametrize("B,CO,CI,G,HW", [(3, 20, 70, 1, 100), (7, 12, 66, 2, 130)])
 def test_backward_conv_layout_many_positions(B, CO, CI, G, HW, p):
