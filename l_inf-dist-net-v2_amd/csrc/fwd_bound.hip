@@ -7,6 +7,7 @@
 
 #include "fwd_tile.h"
 #include "rescan_sorted.h"
+#include "rescan_image.h"
 
 namespace ndist {
 
@@ -254,6 +255,10 @@ int launch_bound_forward(const float* xl, const float* xu, const float* w, const
     }
     if (rc) return done(rc);
     const int imp = cv != nullptr;
+    if (imp && rescan_image_enabled()) {  // images: both second passes on one staged pair of image rows
+        const int r = launch_rescan_image<true>(xl, xu, w, yl, pl, yu, pu, s, kt, st, pm);
+        if (r != -1) return done(r);
+    }
     if (rescan_sorted_applies(s, kt)) {
         const int r1 = launch_rescan_sorted<1>(xl, xu, w, yl, pl, s, kt, st, imp ? &pm : nullptr);
         return done(r1 ? r1 : launch_rescan_sorted<2>(xl, xu, w, yu, pu, s, kt, st, imp ? &pm : nullptr));

@@ -10,6 +10,7 @@
 // very small HW.
 #include "fwd_tile.h"
 #include "rescan_sorted.h"
+#include "rescan_image.h"
 
 namespace ndist {
 
@@ -243,6 +244,10 @@ int launch_inf_forward(const float* x, const float* w, const Geom& s, float* out
         if (!rc && kt2 != kt) rc = 2;  // (same candidate list and cost model: cannot differ)
     }
     if (rc) return done(rc);
+    if (cv != nullptr && rescan_image_enabled()) {  // images: the second pass on staged image rows, where they fit
+        const int r = launch_rescan_image<false>(x, nullptr, w, out, pos, nullptr, nullptr, s, kt, st, pm);
+        if (r != -1) return done(r);
+    }
     if (rescan_sorted_applies(s, kt))
         return done(launch_rescan_sorted<0>(x, nullptr, w, out, pos, s, kt, st, cv ? &pm : nullptr));
     const long total = (long)s.M * s.COg * s.G;

@@ -1,0 +1,228 @@
+// Second pass of the arg-max forward kernels of a convolutional layer called on images: turns the winning k-tile of
+// every output into the arg-max code (reference semantics: core/cuda/inf_dist_cuda.cu:14-198 and
+// core/cuda/bound_inf_dist_cuda.cu:15-238 keep the first k that attains the extremum, plus a sign flag).
+//
+// The sorted second pass (rescan_sorted.h) gathers a k-tile of patches through the patch geometry once per tile and
+// workgroup, 36 times at 3 x 3 windows over 128 channels, with two barriers each.  Here a workgroup owns a few whole
+// output rows of one sample and stages the image rows under their windows ONCE: all channels of the group, padding
+// included as zeros, in LDS (70 KB for two output rows of a 32 x 32 image with 128 channels).  Every patch element
+// of every position of the block is then one LDS read away — its address is a per-k table entry plus a per-position
+// offset — so each output looks at its own winning tile directly: no sort, no barrier after the staging, no atomics.
+// Eight lanes share an output (four consecutive k each, one 128-byte line of the weight row between them); a wave
+// reads tile and target of 64 consecutive positions of one output channel with coalesced loads, hands them to the
+// groups of eight lanes by shuffles, and writes the 64 codes back coalesced.
+//
+// BOUND: both interval outputs in one launch (lower first, then upper) on the same staged pair of images, inverted
+// boxes collapsed to their midpoint while staging (reference: core/cuda/bound_inf_dist_cuda.cu:63).
+#pragma once
+#include "ndist_common.h"
+#include <algorithm>
+#include <cstdlib>
+
+namespace ndist {
+
+constexpr int kRiMaxSlots = 8;               // staged elements of one channel per lane: 64 * 8 floats per channel
+constexpr int kRiLdsBudget = 150 * 1024;     // of the 160 KB of a compute unit
+constexpr int kRiMaxK = 8192;
+
+struct RescanImageGeom {
+    int R;         // output rows per workgroup
+    int nrb;       // row blocks per sample
+    int rows_in;   // image rows staged per channel: (R - 1) sh + (kh - 1) dh + 1
+    int pitch;     // staged row length: W + 2 pw
+    int E;         // rows_in * pitch, floats per channel
+    int nt;        // number of k-tiles
+    float inv_pitch, inv_ow;
+};
+
+template <bool BOUND, int KT>
+__global__ __launch_bounds__(1024) void rescan_image_kernel(const float* __restrict__ x, const float* __restrict__ x2,
+                                                            const float* __restrict__ w, const float* __restrict__ out1,
+                                                            int32_t* __restrict__ pos1, const float* __restrict__ out2,
+                                                            int32_t* __restrict__ pos2, const Geom s, const PatchMap pm,
+                                                            const RescanImageGeom rg, int w_vec) {
+    extern __shared__ float lds[];
+    constexpr int NX = BOUND ? 2 : 1;
+    constexpr uint32_t kNoKey = 0xffffffffu;
+    static_assert(KT == 16 || KT == 32, "eight lanes of four k cover a tile");
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), nwave = (int)blockDim.x >> 6;
+    unsigned id = blockIdx.x;
+    const int rb = (int)(id % (unsigned)rg.nrb);
+    id /= (unsigned)rg.nrb;
+    const int g = (int)(id % (unsigned)s.G), b = (int)(id / (unsigned)s.G);
+    const int cg = pm.cg, E = rg.E, K = s.CIg, OW = pm.OW, OH = s.HW / pm.OW;
+    float* __restrict__ xs = lds;                                                 // [NX][cg][E]
+    int* __restrict__ tab = reinterpret_cast<int*>(lds + (size_t)NX * cg * E);    // [K]: tap of k as an offset in xs
+    const int oh0 = rb * rg.R, nrow = min(rg.R, OH - oh0), npos = nrow * OW, hw0 = oh0 * OW;
+    const int ih_base = oh0 * pm.sh - pm.ph;
+
+    for (int k = tid; k < K; k += (int)blockDim.x) {
+        const int cl = small_div(k, pm.taps, pm.inv_taps), tap = k - cl * pm.taps;
+        const int ti = small_div(tap, pm.kw, pm.inv_kw), tj = tap - ti * pm.kw;
+        tab[k] = cl * E + ti * pm.dh * rg.pitch + tj * pm.dw;
+    }
+    // ---- staging: a wave takes whole channels; what a lane fetches of a channel is the same for every channel
+    {
+        int goff[kRiMaxSlots];
+        bool ok[kRiMaxSlots];
+#pragma unroll
+        for (int q = 0; q < kRiMaxSlots; q++) {
+            const int e = lane + 64 * q;
+            const int r = small_div(e, rg.pitch, rg.inv_pitch), col = e - r * rg.pitch;
+            const int ih = ih_base + r, iw = col - pm.pw;
+            ok[q] = e < E && (unsigned)ih < (unsigned)pm.H && (unsigned)iw < (unsigned)pm.W;
+            goff[q] = ok[q] ? ih * pm.W + iw : 0;
+        }
+        const long plane = (long)pm.H * pm.W;
+        const float* __restrict__ img1 = x + ((long)b * pm.C + (long)g * cg) * plane;
+        const float* __restrict__ img2 = BOUND ? x2 + ((long)b * pm.C + (long)g * cg) * plane : nullptr;
+#pragma unroll 2
+        for (int c = wave; c < cg; c += nwave) {
+            float v1[kRiMaxSlots], v2[kRiMaxSlots];
+#pragma unroll
+            for (int q = 0; q < kRiMaxSlots; q++) {
+                if (64 * q < E) {  // uniform
+                    v1[q] = img1[c * plane + goff[q]];
+                    if (BOUND) v2[q] = img2[c * plane + goff[q]];
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < kRiMaxSlots; q++) {
+                const int e = lane + 64 * q;
+                if (64 * q < E && e < E) {
+                    float lo = ok[q] ? v1[q] : 0.f;
+                    if (BOUND) {
+                        float hi = ok[q] ? v2[q] : 0.f;
+                        if (lo > hi) lo = hi = (lo + hi) * 0.5f;
+                        xs[(cg + c) * E + e] = hi;
+                    }
+                    xs[c * E + e] = lo;
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- every output looks at its winning tile
+    const int nmacro = (npos + 63) >> 6;  // blocks of 64 consecutive positions
+    const int total = s.COg * nmacro;
+#pragma unroll 1
+    for (int side = 0; side < (BOUND ? 2 : 1); side++) {
+        const float* __restrict__ out = side == 0 ? out1 : out2;
+        int32_t* __restrict__ pos = side == 0 ? pos1 : pos2;
+        const bool lower = BOUND && side == 0;
+        const uint32_t kDefault = lower ? kNoGradId : 0u;
+#pragma unroll 1
+        for (int it = wave; it < total; it += nwave) {
+            const int n = it / nmacro, p = (it - n * nmacro) * 64 + lane;
+            const bool live = p < npos;
+            int t = -1, poff = 0;
+            float val = 0.f;
+            long o = 0;
+            if (live) {
+                o = y_off(s, b, g, n, hw0 + p);
+                t = pos[o];
+                const float v = out[o];
+                val = lower ? -v : v;
+                const int pr = small_div(p, OW, rg.inv_ow), pc = p - pr * OW;
+                poff = pr * pm.sh * rg.pitch + pc * pm.sw;
+                if (t < 0 || t >= rg.nt) t = -1;
+            }
+            const float* __restrict__ wrow = w + w_off(s, g, n, 0);
+            const int quad = (lane & 7) * 4;
+            uint32_t mine = kNoKey;  // the result of the output this lane read
+#pragma unroll
+            for (int sub = 0; sub < 8; sub++) {
+                const int src = (lane & ~7) | sub;
+                const int tt = __shfl(t, src, 64), po = __shfl(poff, src, 64);
+                const float target = __shfl(val, src, 64);
+                uint32_t key = kNoKey;
+                const int k = tt * KT + quad;
+                if (tt >= 0 && quad < KT && k < K) {
+                    float wv[4];
+                    if (w_vec) {
+                        const float4 w4 = *reinterpret_cast<const float4*>(wrow + k);
+                        wv[0] = w4.x; wv[1] = w4.y; wv[2] = w4.z; wv[3] = w4.w;
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; j++) wv[j] = k + j < K ? wrow[k + j] : 0.f;
+                    }
+#pragma unroll
+                    for (int j = 3; j >= 0; j--) {  // descending: the lowest matching k is kept
+                        const int kk = min(k + j, K - 1);
+                        const int a = tab[kk] + po;
+                        bool hit, neg;
+                        if constexpr (!BOUND) {
+                            const float d = xs[a] - wv[j];
+                            hit = fabsf(d) == target;
+                            neg = !(d >= 0);
+                        } else {
+                            const float t1 = wv[j] - xs[a], t2 = xs[cg * E + a] - wv[j];
+                            hit = (lower ? fminf(t1, t2) : fmaxf(t1, t2)) == target;
+                            neg = !(t1 <= t2);
+                        }
+                        if (hit && k + j < K) key = ((uint32_t)(k + j) << 1) | (neg ? 1u : 0u);
+                    }
+                }
+                // lowest key of the eight lanes that share the output (all lanes of the wave are here)
+                key = min(key, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)key, 0xB1, 0xf, 0xf, true));   // quad_perm [1,0,3,2]
+                key = min(key, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)key, 0x4E, 0xf, 0xf, true));   // quad_perm [2,3,0,1]
+                key = min(key, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)key, 0x141, 0xf, 0xf, true));  // row_half_mirror
+                if ((lane & 7) == sub) mine = key;
+            }
+            if (live) {
+                uint32_t code = kDefault;
+                if (t >= 0 && mine != kNoKey) code = (mine >> 1) | ((mine & 1u) ? kSignBit : 0u);
+                pos[o] = (int32_t)code;
+            }
+        }
+    }
+}
+
+// tuning aid: NORM_DIST_RESCAN_IMAGE=0 keeps the sorted second pass for images too
+inline bool rescan_image_enabled() {
+    static const char* v = getenv("NORM_DIST_RESCAN_IMAGE");
+    return v == nullptr || v[0] != '0';
+}
+
+// Launches the second pass on staged image rows; -1 when the geometry does not fit (the caller falls back on the
+// sorted second pass).  BOUND: out1 / pos1 are the lower outputs, out2 / pos2 the upper ones.
+template <bool BOUND>
+int launch_rescan_image(const float* x, const float* x2, const float* w, const float* out1, int32_t* pos1,
+                        const float* out2, int32_t* pos2, const Geom& s, int kt, hipStream_t st, const PatchMap& pm) {
+    if (kt != 16 && kt != 32) return -1;
+    const int OW = pm.OW, OH = s.HW / OW, kh = pm.taps / pm.kw;
+    if (OW <= 0 || OH * OW != s.HW || s.CIg > kRiMaxK) return -1;
+    RescanImageGeom rg{};
+    rg.R = OW >= 64 ? 1 : std::min(OH, std::max(1, 64 / OW));
+    rg.rows_in = (rg.R - 1) * pm.sh + (kh - 1) * pm.dh + 1;
+    rg.pitch = pm.W + 2 * pm.pw;
+    const long e = (long)rg.rows_in * rg.pitch;
+    if (e > 64 * kRiMaxSlots) return -1;
+    rg.E = (int)e;
+    rg.nrb = ceil_div(OH, rg.R);
+    rg.nt = ceil_div(s.CIg, kt);
+    rg.inv_pitch = 1.0f / (float)rg.pitch;
+    rg.inv_ow = 1.0f / (float)OW;
+    const size_t lds = ((size_t)(BOUND ? 2 : 1) * pm.cg * rg.E + (size_t)s.CIg) * sizeof(float);
+    if (lds > (size_t)kRiLdsBudget) return -1;
+    const long nwg = (long)s.B * s.G * rg.nrb;
+    if (nwg >= (1L << 31)) return -1;
+    // two 512-thread workgroups per compute unit when their LDS allows it, else one of 1024 threads
+    const int threads = 2 * lds <= (size_t)kRiLdsBudget ? 512 : 1024;
+    const int w_vec = s.CIg % 4 == 0 && (uintptr_t)w % 16 == 0;
+#define NDIST_RESCAN_IMAGE(KT_)                                                                                          \
+    do {                                                                                                                 \
+        NDIST_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&rescan_image_kernel<BOUND, KT_>),               \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, kRiLdsBudget));                    \
+        hipLaunchKernelGGL((rescan_image_kernel<BOUND, KT_>), dim3((unsigned)nwg), dim3(threads), lds, st, x, x2, w, out1, \
+                           pos1, out2, pos2, s, pm, rg, w_vec);                                                          \
+    } while (0)
+    if (kt == 16) NDIST_RESCAN_IMAGE(16);
+    else NDIST_RESCAN_IMAGE(32);
+#undef NDIST_RESCAN_IMAGE
+    return hip_failed(hipGetLastError()) ? 4 : 0;
+}
+
+}  // namespace ndist
