@@ -18,6 +18,7 @@
 #include "ndist_common.h"
 #include <algorithm>
 #include <cstdlib>
+#include <type_traits>
 
 namespace ndist {
 
@@ -35,6 +36,17 @@ struct RescanImageGeom {
     float inv_pitch, inv_ow;
 };
 
+// Value of lane SUB of every group of eight lanes, in all lanes of the group, without the LDS crossbar: the quad that
+// holds the lane spreads it with a quad permutation, the other quad takes it from there through the mirror of the
+// eight lanes.
+template <int SUB>
+__device__ __forceinline__ int group_bcast(int v, int lane) {
+    constexpr int q = SUB & 3, ctrl = q | (q << 2) | (q << 4) | (q << 6);  // quad_perm [q, q, q, q]
+    const int own = __builtin_amdgcn_update_dpp(0, v, ctrl, 0xf, 0xf, true);
+    const int other = __builtin_amdgcn_update_dpp(0, own, 0x141, 0xf, 0xf, true);  // row_half_mirror
+    return ((lane >> 2) & 1) == (SUB >> 2) ? own : other;
+}
+
 template <bool BOUND, int KT>
 __global__ __launch_bounds__(1024) void rescan_image_kernel(const float* __restrict__ x, const float* __restrict__ x2,
                                                             const float* __restrict__ w, const float* __restrict__ out1,
@@ -42,7 +54,6 @@ __global__ __launch_bounds__(1024) void rescan_image_kernel(const float* __restr
                                                             int32_t* __restrict__ pos2, const Geom s, const PatchMap pm,
                                                             const RescanImageGeom rg, int w_vec) {
     extern __shared__ float lds[];
-    constexpr int NX = BOUND ? 2 : 1;
     constexpr uint32_t kNoKey = 0xffffffffu;
     static_assert(KT == 16 || KT == 32, "eight lanes of four k cover a tile");
     const int tid = threadIdx.x, lane = tid & 63;
@@ -52,13 +63,15 @@ __global__ __launch_bounds__(1024) void rescan_image_kernel(const float* __restr
     id /= (unsigned)rg.nrb;
     const int g = (int)(id % (unsigned)s.G), b = (int)(id / (unsigned)s.G);
     const int cg = pm.cg, E = rg.E, K = s.CIg, OW = pm.OW, OH = s.HW / pm.OW;
-    float* __restrict__ xs = lds;                                                 // [NX][cg][E]
-    int* __restrict__ tab = reinterpret_cast<int*>(lds + (size_t)NX * cg * E);    // [K]: tap of k as an offset in xs
+    const int K4 = (K + 3) & ~3;
+    int* __restrict__ tab = reinterpret_cast<int*>(lds);  // [K4]: tap of k as an offset in xs (16-byte aligned)
+    float* __restrict__ xs = lds + K4;                     // [NX][cg][E]
     const int oh0 = rb * rg.R, nrow = min(rg.R, OH - oh0), npos = nrow * OW, hw0 = oh0 * OW;
     const int ih_base = oh0 * pm.sh - pm.ph;
 
-    for (int k = tid; k < K; k += (int)blockDim.x) {
-        const int cl = small_div(k, pm.taps, pm.inv_taps), tap = k - cl * pm.taps;
+    for (int k = tid; k < K4; k += (int)blockDim.x) {
+        const int kc = min(k, K - 1);  // the entries that round K up to whole quads are never used for a hit
+        const int cl = small_div(kc, pm.taps, pm.inv_taps), tap = kc - cl * pm.taps;
         const int ti = small_div(tap, pm.kw, pm.inv_kw), tj = tap - ti * pm.kw;
         tab[k] = cl * E + ti * pm.dh * rg.pitch + tj * pm.dw;
     }
@@ -132,11 +145,10 @@ __global__ __launch_bounds__(1024) void rescan_image_kernel(const float* __restr
             const float* __restrict__ wrow = w + w_off(s, g, n, 0);
             const int quad = (lane & 7) * 4;
             uint32_t mine = kNoKey;  // the result of the output this lane read
-#pragma unroll
-            for (int sub = 0; sub < 8; sub++) {
-                const int src = (lane & ~7) | sub;
-                const int tt = __shfl(t, src, 64), po = __shfl(poff, src, 64);
-                const float target = __shfl(val, src, 64);
+            auto step = [&](auto sub_c) __attribute__((always_inline)) {
+                constexpr int sub = decltype(sub_c)::value;
+                const int tt = group_bcast<sub>(t, lane), po = group_bcast<sub>(poff, lane);
+                const float target = __int_as_float(group_bcast<sub>(__float_as_int(val), lane));
                 uint32_t key = kNoKey;
                 const int k = tt * KT + quad;
                 if (tt >= 0 && quad < KT && k < K) {
@@ -148,17 +160,23 @@ __global__ __launch_bounds__(1024) void rescan_image_kernel(const float* __restr
 #pragma unroll
                         for (int j = 0; j < 4; j++) wv[j] = k + j < K ? wrow[k + j] : 0.f;
                     }
+                    const int4 tp4 = *reinterpret_cast<const int4*>(tab + k);  // (k is a multiple of four)
+                    const int tp[4] = {tp4.x, tp4.y, tp4.z, tp4.w};
+                    float xa[4], xb[4];  // the reads leave together
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        xa[j] = xs[tp[j] + po];
+                        xb[j] = BOUND ? xs[cg * E + tp[j] + po] : 0.f;
+                    }
 #pragma unroll
                     for (int j = 3; j >= 0; j--) {  // descending: the lowest matching k is kept
-                        const int kk = min(k + j, K - 1);
-                        const int a = tab[kk] + po;
                         bool hit, neg;
                         if constexpr (!BOUND) {
-                            const float d = xs[a] - wv[j];
+                            const float d = xa[j] - wv[j];
                             hit = fabsf(d) == target;
                             neg = !(d >= 0);
                         } else {
-                            const float t1 = wv[j] - xs[a], t2 = xs[cg * E + a] - wv[j];
+                            const float t1 = wv[j] - xa[j], t2 = xb[j] - wv[j];
                             hit = (lower ? fminf(t1, t2) : fmaxf(t1, t2)) == target;
                             neg = !(t1 <= t2);
                         }
@@ -170,7 +188,11 @@ __global__ __launch_bounds__(1024) void rescan_image_kernel(const float* __restr
                 key = min(key, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)key, 0x4E, 0xf, 0xf, true));   // quad_perm [2,3,0,1]
                 key = min(key, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)key, 0x141, 0xf, 0xf, true));  // row_half_mirror
                 if ((lane & 7) == sub) mine = key;
-            }
+            };
+            step(std::integral_constant<int, 0>{}); step(std::integral_constant<int, 1>{});
+            step(std::integral_constant<int, 2>{}); step(std::integral_constant<int, 3>{});
+            step(std::integral_constant<int, 4>{}); step(std::integral_constant<int, 5>{});
+            step(std::integral_constant<int, 6>{}); step(std::integral_constant<int, 7>{});
             if (live) {
                 uint32_t code = kDefault;
                 if (t >= 0 && mine != kNoKey) code = (mine >> 1) | ((mine & 1u) ? kSignBit : 0u);
@@ -205,7 +227,7 @@ int launch_rescan_image(const float* x, const float* x2, const float* w, const f
     rg.nt = ceil_div(s.CIg, kt);
     rg.inv_pitch = 1.0f / (float)rg.pitch;
     rg.inv_ow = 1.0f / (float)OW;
-    const size_t lds = ((size_t)(BOUND ? 2 : 1) * pm.cg * rg.E + (size_t)s.CIg) * sizeof(float);
+    const size_t lds = ((size_t)(BOUND ? 2 : 1) * pm.cg * rg.E + (size_t)((s.CIg + 3) & ~3)) * sizeof(float);
     if (lds > (size_t)kRiLdsBudget) return -1;
     const long nwg = (long)s.B * s.G * rg.nrb;
     if (nwg >= (1L << 31)) return -1;
