@@ -204,7 +204,7 @@ __global__ __launch_bounds__(1024) void rescan_image_kernel(const float* __restr
 
 // tuning aid: NORM_DIST_RESCAN_IMAGE=0 keeps the sorted second pass for images too
 inline bool rescan_image_enabled() {
-    static const char* v = getenv("NORM_DIST_RESCAN_IMAGE");
+    const char* v = getenv("NORM_DIST_RESCAN_IMAGE");  // read at every call: the tests switch it
     return v == nullptr || v[0] != '0';
 }
 

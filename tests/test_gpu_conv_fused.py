@@ -70,6 +70,9 @@ TRAIN_CASES = CASES + [
     (1, 2, 150, 150, 3, 1, 3, 1, 1, 1),            # an image plane larger than the scatter kernel's LDS tile: the
                                                    # backward takes the unfolded-gradient + adjoint route
     (2, 64, 8, 8, 16, 1, 3, 1, 1, 1),              # several channel slabs per sample in the image-gradient kernel
+    (1, 3, 6, 200, 5, 1, 3, 1, 1, 1),              # rows too long for the second pass on staged image rows: the
+                                                   # sorted second pass gathers the patches instead
+    (2, 300, 6, 6, 7, 1, 3, 1, 1, 1),              # 300 channels: one workgroup of 1024 threads per compute unit
 ]
 
 
@@ -281,3 +284,31 @@ def test_conv_norm_dist_backward_in_parts_of_the_batch(p, G, stride, monkeypatch
     only_x = torch.full_like(xd, float("nan"))
     _C.conv_norm_dist_backward_input(g.cuda(), xd, wd, out, only_x, G, p, k, 1, 1, stride)
     assert_close(only_x.cpu().numpy(), ex_img, tol=tol_x, what="input-only entry point in parts p=%g" % p)
+
+
+@pytest.mark.parametrize("B,C,H,W,CO,G,k,d,p,s", [CASES[2], CASES[6], CASES[7], CASES[9]])
+def test_conv_codes_with_the_sorted_second_pass(B, C, H, W, CO, G, k, d, p, s, monkeypatch):
+    """The arg-max codes of the image entry points come from one of two second passes (staged image rows where they
+    fit LDS, else the sorted gather of patches); NORM_DIST_RESCAN_IMAGE=0 keeps the second one, which must give the
+    same bits."""
+    from core import _C
+    monkeypatch.setenv("NORM_DIST_RESCAN_IMAGE", "0")
+    x, w = _case(B * 47 + C, B, C, H, W, CO, G, k, d, p, s)
+    patches = F.unfold(x, k, d, p, s)
+    eo, ep = O.inf_dist_forward(patches.numpy(), w.numpy(), G)
+    out = torch.empty(B, CO, patches.size(2), device="cuda")
+    pos = torch.empty_like(out, dtype=torch.int32)
+    _C.conv_inf_dist_forward(x.cuda(), w.cuda(), out, pos, G, k, d, p, s)
+    np.testing.assert_array_equal(out.cpu().numpy(), eo)
+    np.testing.assert_array_equal(pos.cpu().numpy(), ep)
+    radius = torch.rand(x.shape, generator=torch.Generator().manual_seed(8)) * 0.2
+    lower, upper = x - radius, x + radius
+    pl, pu = F.unfold(lower, k, d, p, s), F.unfold(upper, k, d, p, s)
+    el, eu, epl, epu = O.bound_inf_dist_forward(pl.numpy(), pu.numpy(), w.numpy(), G)
+    yl = torch.empty(B, CO, pl.size(2), device="cuda")
+    yu = torch.empty_like(yl)
+    posl = torch.empty_like(yl, dtype=torch.int32)
+    posu = torch.empty_like(posl)
+    _C.conv_bound_inf_dist_forward(lower.cuda(), upper.cuda(), w.cuda(), yl, yu, posl, posu, G, k, d, p, s)
+    np.testing.assert_array_equal(posl.cpu().numpy(), epl)
+    np.testing.assert_array_equal(posu.cpu().numpy(), epu)
