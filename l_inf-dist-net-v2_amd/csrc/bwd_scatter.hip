@@ -17,6 +17,7 @@
 //     patch geometry (taps in the padding are dropped, as the adjoint of the patch extraction would drop them) and
 //     writes the slab once.  The unfolded gradient never exists.
 #include "ndist_common.h"
+#include "rescan_image.h"
 
 namespace ndist {
 
@@ -410,6 +411,105 @@ __global__ __launch_bounds__(kImageThreads) void scatter_gx_image_kernel(
     }
 }
 
+// ---- images, by blocks of output rows -------------------------------------------------------------------
+// A workgroup owns a few whole output rows of one sample (image_row_blocks) and every output channel of the group:
+// the image rows under their windows, all channels, padding included, are a block of LDS in which every code of
+// the workgroup's outputs is ONE float add (a per-k table entry plus a per-position offset) — no code is read by a
+// workgroup that has no use for it, where the slab kernel below reads every code of a sample once per channel slab.
+// Neighbouring row blocks share the image rows between their windows, so the block leaves through global float adds
+// into a gradient cleared beforehand (cells that received nothing, and the padding, are not written).
+template <bool BOUND>
+__global__ __launch_bounds__(1024) void scatter_gx_rowblock_kernel(const float* __restrict__ g1, const float* __restrict__ g2,
+                                                                  const int32_t* __restrict__ p1,
+                                                                  const int32_t* __restrict__ p2, float* __restrict__ gx1,
+                                                                  float* __restrict__ gx2, const Geom s, const PatchMap pm,
+                                                                  const ImageRowBlocks rg) {
+    extern __shared__ float lds[];
+    constexpr int NX = BOUND ? 2 : 1;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), nwave = (int)blockDim.x >> 6, nthr = (int)blockDim.x;
+    unsigned id = blockIdx.x;
+    const int rb = (int)(id % (unsigned)rg.nrb);
+    id /= (unsigned)rg.nrb;
+    const int g = (int)(id % (unsigned)s.G), b = (int)(id / (unsigned)s.G);
+    const int cg = pm.cg, E = rg.E, K = s.CIg, OW = pm.OW, OH = s.HW / pm.OW;
+    const int K4 = (K + 3) & ~3;
+    int* __restrict__ tab = reinterpret_cast<int*>(lds);  // [K4]: tap of k as an offset in the block
+    float* __restrict__ acc = lds + K4;                    // [NX][cg][E]
+    const int oh0 = rb * rg.R, nrow = min(rg.R, OH - oh0), npos = nrow * OW, hw0 = oh0 * OW;
+    const int ih_base = oh0 * pm.sh - pm.ph;
+    for (int k = tid; k < K; k += nthr) {
+        const int cl = small_div(k, pm.taps, pm.inv_taps), tap = k - cl * pm.taps;
+        const int ti = small_div(tap, pm.kw, pm.inv_kw), tj = tap - ti * pm.kw;
+        tab[k] = cl * E + ti * pm.dh * rg.pitch + tj * pm.dw;
+    }
+    for (int i = tid; i < NX * cg * E; i += nthr) acc[i] = 0.f;
+    __syncthreads();
+
+    const int nmacro = (npos + 63) >> 6;  // blocks of 64 consecutive positions of one output channel
+    const int total = s.COg * nmacro;
+    constexpr int UN = 4;  // steps whose codes and gradients are requested together
+#pragma unroll 1
+    for (int it0 = wave; it0 < total; it0 += nwave * UN) {
+        int32_t c1[UN], c2[UN];
+        float v1[UN], v2[UN];
+        int poff[UN];
+#pragma unroll
+        for (int u = 0; u < UN; u++) {
+            const int it = it0 + u * nwave;
+            const int n = it / nmacro, p = (it - n * nmacro) * 64 + lane;
+            const bool live = it < total && p < npos;
+            const long o = live ? y_off(s, b, g, n, hw0 + p) : 0;
+            c1[u] = live ? p1[o] : (BOUND ? (int32_t)kNoGradId : 0);
+            v1[u] = live ? g1[o] : 0.f;
+            if (BOUND) {
+                c2[u] = live ? p2[o] : 0;
+                v2[u] = live ? g2[o] : 0.f;
+            }
+            const int pr = small_div(p, OW, rg.inv_ow), pc = p - pr * OW;
+            poff[u] = live ? pr * pm.sh * rg.pitch + pc * pm.sw : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < UN; u++) {
+            if (poff[u] < 0) continue;
+            const Route a = BOUND ? route_lower(c1[u], v1[u]) : route_inf(c1[u], v1[u]);
+            if (a.target >= 0 && a.idx < K && a.v != 0.f) atomicAdd(&acc[a.target * cg * E + tab[a.idx] + poff[u]], a.v);
+            if (BOUND) {
+                const Route c = route_upper(c2[u], v2[u]);
+                if (c.idx < K && c.v != 0.f) atomicAdd(&acc[c.target * cg * E + tab[c.idx] + poff[u]], c.v);
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- the block into the image gradient: a wave takes whole channels, as the staging of the second pass does
+    int goff[kRiMaxSlots];
+    bool ok[kRiMaxSlots];
+#pragma unroll
+    for (int q = 0; q < kRiMaxSlots; q++) {
+        const int e = lane + 64 * q;
+        const int r = small_div(e, rg.pitch, rg.inv_pitch), col = e - r * rg.pitch;
+        const int ih = ih_base + r, iw = col - pm.pw;
+        ok[q] = e < E && (unsigned)ih < (unsigned)pm.H && (unsigned)iw < (unsigned)pm.W;
+        goff[q] = ok[q] ? ih * pm.W + iw : 0;
+    }
+    const long plane = (long)pm.H * pm.W;
+    const long img = ((long)b * pm.C + (long)g * cg) * plane;
+    for (int c = wave; c < cg; c += nwave) {
+#pragma unroll
+        for (int q = 0; q < kRiMaxSlots; q++) {
+            if (64 * q < E && ok[q]) {
+                const float a = acc[c * E + lane + 64 * q];
+                if (a != 0.f) atomicAdd(gx1 + img + c * plane + goff[q], a);
+                if (BOUND) {
+                    const float a2 = acc[(cg + c) * E + lane + 64 * q];
+                    if (a2 != 0.f) atomicAdd(gx2 + img + c * plane + goff[q], a2);
+                }
+            }
+        }
+    }
+}
+
 constexpr int kScatterLdsBudget = 96 * 1024;
 constexpr int kScatterTileBudget = 72 * 1024;  // two workgroups per CU
 
@@ -421,18 +521,10 @@ static int scatter_backward_images(const float* g1, const float* g2, const int32
     const int nx = BOUND ? 2 : 1;
     const long plane = (long)pm.H * pm.W;
     const long fixed = (long)s.HW * 4, per_ch = nx * plane * 4;
-    if (pm.ph >= 8192 || pm.pw >= 8192) return -1;  // window origins are packed into 16 bits (the plane bound limits H, W)
-    if (fixed + per_ch > kScatterTileBudget) return -1;
     if (gw && (size_t)s.CIg * sizeof(float) > (size_t)kScatterLdsBudget) return -1;
-    int CS = (int)((kScatterTileBudget - fixed) / per_ch);
-    CS = CS > pm.cg ? pm.cg : CS;
-    const int nslab = ceil_div(pm.cg, CS);
-    const long nwg = (long)s.B * s.G * nslab;
-    if (nslab > 16 || nwg >= (1L << 31)) return -1;
-    NDIST_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&scatter_gx_image_kernel<BOUND>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, kScatterTileBudget));
+    // grad_weight launch parameters (shared by both grad_input routes)
     int R = 1, ncb = 0, nsplit = 1;
-    if (gw) {
+    auto prepare_gw = [&]() -> int {
         NDIST_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&scatter_gw_split_kernel<BOUND>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, kScatterLdsBudget));
         R = (int)((size_t)kScatterLdsBudget / ((size_t)s.CIg * sizeof(float)));
@@ -441,21 +533,53 @@ static int scatter_backward_images(const float* g1, const float* g2, const int32
         nsplit = ceil_div(4 * device_info().num_cu, ncb * s.G);
         nsplit = nsplit > s.B ? s.B : nsplit;
         nsplit = nsplit > 65535 ? 65535 : nsplit;
-        if (nsplit > 1) {
-            const int rc = fill_zero(gw, (long)s.COg * s.G * s.CIg, st);
+        return nsplit > 1 ? fill_zero(gw, (long)s.COg * s.G * s.CIg, st) : 0;
+    };
+    auto launch_gw = [&]() -> int {
+        hipLaunchKernelGGL(scatter_gw_split_kernel<BOUND>, dim3(ncb, s.G, nsplit), dim3(256),
+                           (size_t)R * s.CIg * sizeof(float), st, g1, g2, p1, p2, gw, s, R, nsplit);
+        return hip_failed(hipGetLastError()) ? 4 : 0;
+    };
+    // by blocks of output rows where the rows under a block fit LDS (tuning aid: NORM_DIST_SCATTER_ROWBLOCKS=0 keeps
+    // the slab kernel)
+    {
+        ImageRowBlocks rg{};
+        size_t lds = 0;
+        const char* sw = getenv("NORM_DIST_SCATTER_ROWBLOCKS");
+        if ((sw == nullptr || sw[0] != '0') && image_row_blocks(s, pm, nx, &rg, &lds)) {
+            NDIST_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&scatter_gx_rowblock_kernel<BOUND>),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, kRiLdsBudget));
+            if (gw) {
+                if (int rc = prepare_gw()) return rc;
+            }
+            int rc = fill_zero(gx1, (long)s.B * pm.C * plane, st);
+            if (!rc && BOUND) rc = fill_zero(gx2, (long)s.B * pm.C * plane, st);
             if (rc) return rc;
+            KernelTimer timer(st);  // both kernels together
+            const int threads = 2 * lds <= (size_t)kRiLdsBudget ? 512 : 1024;
+            hipLaunchKernelGGL(scatter_gx_rowblock_kernel<BOUND>, dim3((unsigned)((long)s.B * s.G * rg.nrb)), dim3(threads),
+                               lds, st, g1, g2, p1, p2, gx1, gx2, s, pm, rg);
+            if (hip_failed(hipGetLastError())) return 4;
+            return gw ? launch_gw() : 0;
         }
+    }
+    if (pm.ph >= 8192 || pm.pw >= 8192) return -1;  // window origins are packed into 16 bits (the plane bound limits H, W)
+    if (fixed + per_ch > kScatterTileBudget) return -1;
+    int CS = (int)((kScatterTileBudget - fixed) / per_ch);
+    CS = CS > pm.cg ? pm.cg : CS;
+    const int nslab = ceil_div(pm.cg, CS);
+    const long nwg = (long)s.B * s.G * nslab;
+    if (nslab > 16 || nwg >= (1L << 31)) return -1;
+    NDIST_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&scatter_gx_image_kernel<BOUND>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, kScatterTileBudget));
+    if (gw) {
+        if (int rc = prepare_gw()) return rc;
     }
     KernelTimer timer(st);  // both kernels together
     hipLaunchKernelGGL(scatter_gx_image_kernel<BOUND>, dim3((unsigned)nwg), dim3(kImageThreads),
                        (size_t)(fixed + (long)CS * per_ch), st, g1, g2, p1, p2, gx1, gx2, s, pm, CS, nslab);
     if (hip_failed(hipGetLastError())) return 4;
-    if (gw) {
-        hipLaunchKernelGGL(scatter_gw_split_kernel<BOUND>, dim3(ncb, s.G, nsplit), dim3(256),
-                           (size_t)R * s.CIg * sizeof(float), st, g1, g2, p1, p2, gw, s, R, nsplit);
-        if (hip_failed(hipGetLastError())) return 4;
-    }
-    return 0;
+    return gw ? launch_gw() : 0;
 }
 
 template <bool BOUND>

@@ -26,7 +26,7 @@ constexpr int kRiMaxSlots = 8;               // staged elements of one channel p
 constexpr int kRiLdsBudget = 150 * 1024;     // of the 160 KB of a compute unit
 constexpr int kRiMaxK = 8192;
 
-struct RescanImageGeom {
+struct ImageRowBlocks {
     int R;         // output rows per workgroup
     int nrb;       // row blocks per sample
     int rows_in;   // image rows staged per channel: (R - 1) sh + (kh - 1) dh + 1
@@ -52,7 +52,7 @@ __global__ __launch_bounds__(1024) void rescan_image_kernel(const float* __restr
                                                             const float* __restrict__ w, const float* __restrict__ out1,
                                                             int32_t* __restrict__ pos1, const float* __restrict__ out2,
                                                             int32_t* __restrict__ pos2, const Geom s, const PatchMap pm,
-                                                            const RescanImageGeom rg, int w_vec) {
+                                                            const ImageRowBlocks rg, int w_vec) {
     extern __shared__ float lds[];
     constexpr uint32_t kNoKey = 0xffffffffu;
     static_assert(KT == 16 || KT == 32, "eight lanes of four k cover a tile");
@@ -202,6 +202,30 @@ __global__ __launch_bounds__(1024) void rescan_image_kernel(const float* __restr
     }
 }
 
+// Row blocks of the image kernels (second pass here, the gradient scatter of bwd_scatter.hip): `arrays` staged copies
+// of the image rows under a block of output rows, plus the table of taps.  False when they do not fit.
+inline bool image_row_blocks(const Geom& s, const PatchMap& pm, int arrays, ImageRowBlocks* out, size_t* lds_bytes) {
+    const int OW = pm.OW, OH = OW > 0 ? s.HW / OW : 0, kh = pm.taps / pm.kw;
+    if (OW <= 0 || OH * OW != s.HW || s.CIg > kRiMaxK) return false;
+    ImageRowBlocks rg{};
+    rg.R = OW >= 64 ? 1 : std::min(OH, std::max(1, 64 / OW));
+    rg.rows_in = (rg.R - 1) * pm.sh + (kh - 1) * pm.dh + 1;
+    rg.pitch = pm.W + 2 * pm.pw;
+    const long e = (long)rg.rows_in * rg.pitch;
+    if (e > 64 * kRiMaxSlots) return false;
+    rg.E = (int)e;
+    rg.nrb = ceil_div(OH, rg.R);
+    rg.nt = 0;
+    rg.inv_pitch = 1.0f / (float)rg.pitch;
+    rg.inv_ow = 1.0f / (float)OW;
+    const size_t lds = ((size_t)arrays * pm.cg * rg.E + (size_t)((s.CIg + 3) & ~3)) * sizeof(float);
+    if (lds > (size_t)kRiLdsBudget) return false;
+    if ((long)s.B * s.G * rg.nrb >= (1L << 31)) return false;
+    *out = rg;
+    *lds_bytes = lds;
+    return true;
+}
+
 // tuning aid: NORM_DIST_RESCAN_IMAGE=0 keeps the sorted second pass for images too
 inline bool rescan_image_enabled() {
     const char* v = getenv("NORM_DIST_RESCAN_IMAGE");  // read at every call: the tests switch it
@@ -214,23 +238,11 @@ template <bool BOUND>
 int launch_rescan_image(const float* x, const float* x2, const float* w, const float* out1, int32_t* pos1,
                         const float* out2, int32_t* pos2, const Geom& s, int kt, hipStream_t st, const PatchMap& pm) {
     if (kt != 16 && kt != 32) return -1;
-    const int OW = pm.OW, OH = s.HW / OW, kh = pm.taps / pm.kw;
-    if (OW <= 0 || OH * OW != s.HW || s.CIg > kRiMaxK) return -1;
-    RescanImageGeom rg{};
-    rg.R = OW >= 64 ? 1 : std::min(OH, std::max(1, 64 / OW));
-    rg.rows_in = (rg.R - 1) * pm.sh + (kh - 1) * pm.dh + 1;
-    rg.pitch = pm.W + 2 * pm.pw;
-    const long e = (long)rg.rows_in * rg.pitch;
-    if (e > 64 * kRiMaxSlots) return -1;
-    rg.E = (int)e;
-    rg.nrb = ceil_div(OH, rg.R);
+    ImageRowBlocks rg{};
+    size_t lds = 0;
+    if (!image_row_blocks(s, pm, BOUND ? 2 : 1, &rg, &lds)) return -1;
     rg.nt = ceil_div(s.CIg, kt);
-    rg.inv_pitch = 1.0f / (float)rg.pitch;
-    rg.inv_ow = 1.0f / (float)OW;
-    const size_t lds = ((size_t)(BOUND ? 2 : 1) * pm.cg * rg.E + (size_t)((s.CIg + 3) & ~3)) * sizeof(float);
-    if (lds > (size_t)kRiLdsBudget) return -1;
     const long nwg = (long)s.B * s.G * rg.nrb;
-    if (nwg >= (1L << 31)) return -1;
     // two 512-thread workgroups per compute unit when their LDS allows it, else one of 1024 threads
     const int threads = 2 * lds <= (size_t)kRiLdsBudget ? 512 : 1024;
     const int w_vec = s.CIg % 4 == 0 && (uintptr_t)w % 16 == 0;

@@ -312,3 +312,37 @@ def test_conv_codes_with_the_sorted_second_pass(B, C, H, W, CO, G, k, d, p, s, m
     _C.conv_bound_inf_dist_forward(lower.cuda(), upper.cuda(), w.cuda(), yl, yu, posl, posu, G, k, d, p, s)
     np.testing.assert_array_equal(posl.cpu().numpy(), epl)
     np.testing.assert_array_equal(posu.cpu().numpy(), epu)
+
+
+@pytest.mark.parametrize("B,C,H,W,CO,G,k,d,p,s", [CASES[2], CASES[6], CASES[7], TRAIN_CASES[-1]])
+def test_conv_backward_by_channel_slabs(B, C, H, W, CO, G, k, d, p, s, monkeypatch):
+    """The image gradient of the scatter backward comes from one of two kernels (blocks of output rows where the image
+    rows under a block fit LDS, else slabs of channels); NORM_DIST_SCATTER_ROWBLOCKS=0 keeps the second one: same
+    gradients within 1e-5 of the oracle, for the distance and for the interval bounds."""
+    from core import _C
+    x, w = _case(B * 53 + C, B, C, H, W, CO, G, k, d, p, s)
+    x *= 0.3
+    radius = torch.rand(x.shape, generator=torch.Generator().manual_seed(9)) * 0.2
+    lower, upper = x - radius, x + radius
+    patches, pl, pu = F.unfold(x, k, d, p, s), F.unfold(lower, k, d, p, s), F.unfold(upper, k, d, p, s)
+    _, ep = O.inf_dist_forward(patches.numpy(), w.numpy(), G)
+    _, _, epl, epu = O.bound_inf_dist_forward(pl.numpy(), pu.numpy(), w.numpy(), G)
+    gen = torch.Generator().manual_seed(10)
+    g, gl, gu = (torch.randn(ep.shape, generator=gen) for _ in range(3))
+    ex_p, ew = O.inf_dist_backward(g.numpy(), ep, patches.size(1), G)
+    exl_p, exu_p, ewb = O.bound_inf_dist_backward(gl.numpy(), gu.numpy(), epl, epu, pl.size(1), G)
+    ex, exl, exu = (_fold(t, x.shape, k, d, p, s) for t in (ex_p, exl_p, exu_p))
+    pos, posl, posu = (torch.from_numpy(t).cuda() for t in (ep, epl, epu))
+    for mode in ("1", "0"):
+        monkeypatch.setenv("NORM_DIST_SCATTER_ROWBLOCKS", mode)
+        gx = torch.full(x.shape, float("nan"), device="cuda")
+        gw = torch.full(w.shape, float("nan"), device="cuda")
+        _C.conv_inf_dist_backward_input_weight(g.cuda(), pos, gx, gw, G, k, d, p, s)
+        assert_close(gx.cpu().numpy(), ex, what="grad_input, row blocks " + mode)
+        assert_close(gw.cpu().numpy(), ew, what="grad_weight, row blocks " + mode)
+        gxl = torch.full(x.shape, float("nan"), device="cuda")
+        gxu = torch.full(x.shape, float("nan"), device="cuda")
+        _C.conv_bound_inf_dist_backward_input_weight(gl.cuda(), gu.cuda(), posl, posu, gxl, gxu, gw, G, k, d, p, s)
+        assert_close(gxl.cpu().numpy(), exl, what="grad_lower, row blocks " + mode)
+        assert_close(gxu.cpu().numpy(), exu, what="grad_upper, row blocks " + mode)
+        assert_close(gw.cpu().numpy(), ewb, what="grad_weight (bounds), row blocks " + mode)
