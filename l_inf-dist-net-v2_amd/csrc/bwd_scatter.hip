@@ -510,6 +510,107 @@ __global__ __launch_bounds__(1024) void scatter_gx_rowblock_kernel(const float* 
     }
 }
 
+// The same by blocks of IMAGE rows: a workgroup owns RI whole rows of every channel of one sample's group, reads the
+// codes of all output rows whose windows touch them (the rows between two blocks are read by both: (RI + reach) / RI
+// times the codes, reach = (kh - 1) dh rows), keeps the adds that land in its rows and writes them once, coalesced:
+// no global atomics, no cleared gradient.  A tap is one table word (channel << 16 | dy << 8 | dx).
+struct ImageRowOwners {
+    int RI;    // image rows per workgroup
+    int nib;   // row blocks per sample
+    float inv_ow;
+};
+template <bool BOUND>
+__global__ __launch_bounds__(1024) void scatter_gx_ownrows_kernel(const float* __restrict__ g1, const float* __restrict__ g2,
+                                                                 const int32_t* __restrict__ p1,
+                                                                 const int32_t* __restrict__ p2, float* __restrict__ gx1,
+                                                                 float* __restrict__ gx2, const Geom s, const PatchMap pm,
+                                                                 const ImageRowOwners ro) {
+    extern __shared__ float lds[];
+    constexpr int NX = BOUND ? 2 : 1;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), nwave = (int)blockDim.x >> 6, nthr = (int)blockDim.x;
+    unsigned id = blockIdx.x;
+    const int ib = (int)(id % (unsigned)ro.nib);
+    id /= (unsigned)ro.nib;
+    const int g = (int)(id % (unsigned)s.G), b = (int)(id / (unsigned)s.G);
+    const int cg = pm.cg, K = s.CIg, OW = pm.OW, OH = s.HW / pm.OW, W = pm.W, RI = ro.RI;
+    const int K4 = (K + 3) & ~3, kh = pm.taps / pm.kw;
+    int* __restrict__ tab = reinterpret_cast<int*>(lds);  // [K4]
+    float* __restrict__ acc = lds + K4;                    // [NX][cg][RI][W]
+    const int r0 = ib * RI, rows = min(RI, pm.H - r0), cell = RI * W;
+    // output rows whose windows reach the rows [r0, r0 + rows)
+    const int lo_num = r0 + pm.ph - (kh - 1) * pm.dh;
+    const int oh_lo = lo_num <= 0 ? 0 : (lo_num + pm.sh - 1) / pm.sh;
+    const int oh_hi = min(OH - 1, (r0 + rows - 1 + pm.ph) / pm.sh);
+    const int npos = oh_hi >= oh_lo ? (oh_hi - oh_lo + 1) * OW : 0, hw0 = oh_lo * OW;
+    for (int k = tid; k < K; k += nthr) tab[k] = pack_tap(patch_tap(pm, 0, k));
+    for (int i = tid; i < NX * cg * cell; i += nthr) acc[i] = 0.f;
+    __syncthreads();
+
+    const int nmacro = (npos + 63) >> 6;
+    const int total = s.COg * nmacro;
+    constexpr int UN = 4;
+    auto add = [&](const Route& a, int rowbase, int colbase) __attribute__((always_inline)) {
+        if (a.target < 0 || a.idx >= K || a.v == 0.f) return;
+        const PatchTap t = unpack_tap(tab[a.idx]);
+        const int row = rowbase + t.dy, col = colbase + t.dx;
+        if ((unsigned)row < (unsigned)rows && (unsigned)col < (unsigned)W)
+            atomicAdd(&acc[(a.target * cg + t.ch) * cell + row * W + col], a.v);
+    };
+#pragma unroll 1
+    for (int it0 = wave; it0 < total; it0 += nwave * UN) {
+        int32_t c1[UN], c2[UN];
+        float v1[UN], v2[UN];
+        int rowbase[UN], colbase[UN];
+        bool live[UN];
+#pragma unroll
+        for (int u = 0; u < UN; u++) {
+            const int it = it0 + u * nwave;
+            const int n = it / nmacro, p = (it - n * nmacro) * 64 + lane;
+            live[u] = it < total && p < npos;
+            const long o = live[u] ? y_off(s, b, g, n, hw0 + p) : 0;
+            c1[u] = live[u] ? p1[o] : (BOUND ? (int32_t)kNoGradId : 0);
+            v1[u] = live[u] ? g1[o] : 0.f;
+            if (BOUND) {
+                c2[u] = live[u] ? p2[o] : 0;
+                v2[u] = live[u] ? g2[o] : 0.f;
+            }
+            const int pr = small_div(p, OW, ro.inv_ow), pc = p - pr * OW;
+            rowbase[u] = (oh_lo + pr) * pm.sh - pm.ph - r0;
+            colbase[u] = pc * pm.sw - pm.pw;
+        }
+#pragma unroll
+        for (int u = 0; u < UN; u++) {
+            if (!live[u]) continue;
+            add(BOUND ? route_lower(c1[u], v1[u]) : route_inf(c1[u], v1[u]), rowbase[u], colbase[u]);
+            if (BOUND) add(route_upper(c2[u], v2[u]), rowbase[u], colbase[u]);
+        }
+    }
+    __syncthreads();
+    // ---- my rows of every channel: rows * W contiguous floats per channel
+    const long plane = (long)pm.H * W;
+    const long img = ((long)b * pm.C + (long)g * cg) * plane + (long)r0 * W;
+    const int n = rows * W;
+    const bool vec = n % 4 == 0 && cell % 4 == 0 && plane % 4 == 0 && (r0 * W) % 4 == 0 && (uintptr_t)gx1 % 16 == 0 &&
+                     (!BOUND || (uintptr_t)gx2 % 16 == 0);
+    if (vec) {
+        const int n4 = n / 4;
+        for (int i = tid; i < cg * n4; i += nthr) {
+            const int c = i / n4, e = (i - c * n4) * 4;
+            *reinterpret_cast<float4*>(gx1 + img + c * plane + e) = *reinterpret_cast<const float4*>(acc + c * cell + e);
+            if (BOUND)
+                *reinterpret_cast<float4*>(gx2 + img + c * plane + e) =
+                    *reinterpret_cast<const float4*>(acc + (cg + c) * cell + e);
+        }
+    } else {
+        for (int i = tid; i < cg * n; i += nthr) {
+            const int c = i / n, e = i - c * n;
+            gx1[img + c * plane + e] = acc[c * cell + e];
+            if (BOUND) gx2[img + c * plane + e] = acc[(cg + c) * cell + e];
+        }
+    }
+}
+
 constexpr int kScatterLdsBudget = 96 * 1024;
 constexpr int kScatterTileBudget = 72 * 1024;  // two workgroups per CU
 
@@ -540,12 +641,41 @@ static int scatter_backward_images(const float* g1, const float* g2, const int32
                            (size_t)R * s.CIg * sizeof(float), st, g1, g2, p1, p2, gw, s, R, nsplit);
         return hip_failed(hipGetLastError()) ? 4 : 0;
     };
-    // by blocks of output rows where the rows under a block fit LDS (tuning aid: NORM_DIST_SCATTER_ROWBLOCKS=0 keeps
-    // the slab kernel)
+    // Tuning / test aid: NORM_DIST_SCATTER_ROWBLOCKS=0 keeps the slab kernel, =1 the blocks of output rows.
+    const char* sw = getenv("NORM_DIST_SCATTER_ROWBLOCKS");
+    // By blocks of image rows, where a block can be at least twice as high as the windows reach (at most 1.5 times
+    // the codes read) and a tap packs into a word: two workgroups per compute unit if that height fits half the LDS,
+    // else one of 1024 threads.
+    if ((sw == nullptr || (sw[0] != '0' && sw[0] != '1')) && pm.packable && s.CIg <= kRiMaxK && pm.OW > 0) {
+        const int kh = pm.taps / pm.kw, reach = (kh - 1) * pm.dh;
+        const size_t tabb = (size_t)((s.CIg + 3) & ~3) * sizeof(float);
+        const size_t per_row = (size_t)nx * pm.cg * pm.W * sizeof(float);
+        const int want = std::max(2 * reach, 1);
+        int RI = (int)(((size_t)kRiLdsBudget / 2 - tabb) / per_row), threads = 512;
+        if (RI < want) {
+            RI = (int)(((size_t)kRiLdsBudget - tabb) / per_row);
+            threads = 1024;
+        }
+        RI = std::min(RI, pm.H);
+        const long nwg = RI > 0 ? (long)s.B * s.G * ceil_div(pm.H, RI) : 0;
+        if ((RI >= want || RI == pm.H) && RI > 0 && nwg < (1L << 31)) {
+            const ImageRowOwners ro{RI, ceil_div(pm.H, RI), 1.0f / (float)pm.OW};
+            NDIST_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&scatter_gx_ownrows_kernel<BOUND>),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, kRiLdsBudget));
+            if (gw) {
+                if (int rc = prepare_gw()) return rc;
+            }
+            KernelTimer timer(st);  // both kernels together
+            hipLaunchKernelGGL(scatter_gx_ownrows_kernel<BOUND>, dim3((unsigned)nwg), dim3(threads),
+                               tabb + (size_t)RI * per_row, st, g1, g2, p1, p2, gx1, gx2, s, pm, ro);
+            if (hip_failed(hipGetLastError())) return 4;
+            return gw ? launch_gw() : 0;
+        }
+    }
+    // by blocks of output rows where the rows under a block fit LDS
     {
         ImageRowBlocks rg{};
         size_t lds = 0;
-        const char* sw = getenv("NORM_DIST_SCATTER_ROWBLOCKS");
         if ((sw == nullptr || sw[0] != '0') && image_row_blocks(s, pm, nx, &rg, &lds)) {
             NDIST_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&scatter_gx_rowblock_kernel<BOUND>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, kRiLdsBudget));

@@ -200,10 +200,12 @@ struct UnfoldGeom {
 struct PatchMap {
     int C, H, W, OW, kw, taps, dh, dw, sh, sw, ph, pw, cg;  // taps = kh * kw, cg = image channels per group
     float inv_taps, inv_kw;
+    int packable;  // a tap fits one word: channel inside the group below 2^16, pixel offsets below 2^8 each
 };
 inline PatchMap make_patch_map(const UnfoldGeom& u, int G) {
+    const bool packable = u.C / G < (1 << 16) && (u.kh - 1) * (long)u.dh < 256 && (u.kw - 1) * (long)u.dw < 256;
     return PatchMap{u.C, u.H, u.W, u.OW, u.kw, u.kh * u.kw, u.dh, u.dw, u.sh, u.sw, u.ph, u.pw, u.C / G,
-                    1.0f / (float)(u.kh * u.kw), 1.0f / (float)u.kw};
+                    1.0f / (float)(u.kh * u.kw), 1.0f / (float)u.kw, packable ? 1 : 0};
 }
 
 // floor(a / d) for 0 <= a < 2^22 and 0 < d, with inv = 1.0f / d: the float product is off by at most one
@@ -242,6 +244,11 @@ __device__ __forceinline__ float patch_elem(const float* __restrict__ x, const P
     patch_origin(c, hw, ih0, iw0);
     const long o = patch_offset(c, b, t, ih0, iw0);
     return o >= 0 ? x[o] : 0.f;
+}
+// A tap in one word, for tables of taps in LDS (PatchMap::packable): channel << 16 | dy << 8 | dx.
+__device__ __forceinline__ int pack_tap(const PatchTap& t) { return (t.ch << 16) | (t.dy << 8) | t.dx; }
+__device__ __forceinline__ PatchTap unpack_tap(int v) {
+    return PatchTap{(int)((unsigned)v >> 16), (v >> 8) & 0xff, v & 0xff};
 }
 // four consecutive positions of one output row; (ih0, iw0) is the window origin of the first
 __device__ __forceinline__ float4 patch_row4(const float* __restrict__ x, const PatchMap& c, int b, const PatchTap& t,

@@ -333,7 +333,7 @@ def test_conv_backward_by_channel_slabs(B, C, H, W, CO, G, k, d, p, s, monkeypat
     exl_p, exu_p, ewb = O.bound_inf_dist_backward(gl.numpy(), gu.numpy(), epl, epu, pl.size(1), G)
     ex, exl, exu = (_fold(t, x.shape, k, d, p, s) for t in (ex_p, exl_p, exu_p))
     pos, posl, posu = (torch.from_numpy(t).cuda() for t in (ep, epl, epu))
-    for mode in ("1", "0"):
+    for mode in ("2", "1", "0"):  # blocks of image rows (the default where they fit), of output rows, channel slabs
         monkeypatch.setenv("NORM_DIST_SCATTER_ROWBLOCKS", mode)
         gx = torch.full(x.shape, float("nan"), device="cuda")
         gw = torch.full(w.shape, float("nan"), device="cuda")
