@@ -10,7 +10,7 @@
 // offset — so each output looks at its own winning tile directly: no sort, no barrier after the staging, no atomics.
 // Eight lanes share an output (four consecutive k each, one 128-byte line of the weight row between them); a wave
 // reads tile and target of 64 consecutive positions of one output channel with coalesced loads, hands them to the
-// groups of eight lanes by shuffles, and writes the 64 codes back coalesced.
+// groups of eight lanes by DPP broadcasts (no trip through the LDS crossbar), and writes the 64 codes back coalesced.
 //
 // BOUND: both interval outputs in one launch (lower first, then upper) on the same staged pair of images, inverted
 // boxes collapsed to their midpoint while staging (reference: core/cuda/bound_inf_dist_cuda.cu:63).
