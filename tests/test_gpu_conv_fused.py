@@ -314,11 +314,13 @@ def test_conv_codes_with_the_sorted_second_pass(B, C, H, W, CO, G, k, d, p, s, m
     np.testing.assert_array_equal(posu.cpu().numpy(), epu)
 
 
-@pytest.mark.parametrize("B,C,H,W,CO,G,k,d,p,s", [CASES[2], CASES[6], CASES[7], TRAIN_CASES[-1]])
+@pytest.mark.parametrize("B,C,H,W,CO,G,k,d,p,s", [CASES[2], CASES[6], CASES[7], TRAIN_CASES[-1], TRAIN_CASES[len(CASES)]])
 def test_conv_backward_by_channel_slabs(B, C, H, W, CO, G, k, d, p, s, monkeypatch):
     """The image gradient of the scatter backward comes from one of two kernels (blocks of output rows where the image
     rows under a block fit LDS, else slabs of channels); NORM_DIST_SCATTER_ROWBLOCKS=0 keeps the second one: same
-    gradients within 1e-5 of the oracle, for the distance and for the interval bounds."""
+    gradients within 1e-5 of the oracle, for the distance and for the interval bounds.  The 150 x 150 image fits no
+    slab: with the row kernels switched off its gradient goes through the unfolded gradient and the adjoint of the
+    patch extraction."""
     from core import _C
     x, w = _case(B * 53 + C, B, C, H, W, CO, G, k, d, p, s)
     x *= 0.3
