@@ -185,6 +185,7 @@ bool patch_rows_applies(const UnfoldGeom& u) {
     const int taps = u.kh * u.kw;
     int CC = 8192 / (u.kh * (u.W | 1));
     CC = CC > u.C ? u.C : CC;
+    if (CC >= 4 && CC < u.C) CC &= ~3;
     if (CC < 1 || (long)u.kh * CC * u.W >= (1L << 22) || (long)u.OW * CC * taps >= (1L << 22)) return false;
     return (long)u.B * u.OH * ((u.C + CC - 1) / CC) < (1L << 31);
 }
@@ -194,6 +195,7 @@ int launch_patch_rows(const float* x, const UnfoldGeom& u, float* out, hipStream
     const int taps = u.kh * u.kw;
     int CC = 8192 / (u.kh * (u.W | 1));  // 32 KB of LDS for the strip
     CC = CC > u.C ? u.C : CC;
+    if (CC >= 4 && CC < u.C) CC &= ~3;  // whole quads of channels: every run of a workgroup then allows 16-byte stores
     if (CC < 1 || (long)u.kh * CC * u.W >= (1L << 22) || (long)u.OW * CC * taps >= (1L << 22)) return -1;
     const int ncb = (u.C + CC - 1) / CC;
     const long blocks = (long)u.B * u.OH * ncb;
