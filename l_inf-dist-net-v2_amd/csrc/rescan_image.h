@@ -8,9 +8,9 @@
 // included as zeros, in LDS (70 KB for two output rows of a 32 x 32 image with 128 channels).  Every patch element
 // of every position of the block is then one LDS read away — its address is a per-k table entry plus a per-position
 // offset — so each output looks at its own winning tile directly: no sort, no barrier after the staging, no atomics.
-// Eight lanes share an output (four consecutive k each, one 128-byte line of the weight row between them); a wave
-// reads tile and target of 64 consecutive positions of one output channel with coalesced loads, hands them to the
-// groups of eight lanes by DPP broadcasts (no trip through the LDS crossbar), and writes the 64 codes back coalesced.
+// Four lanes (a quad) share an output: four consecutive k each, twice for tiles of 32 k.  A wave reads tile and target
+// of 64 consecutive positions of one output channel with coalesced loads, hands them to its quads by quad
+// permutations (no trip through the LDS crossbar), and writes the 64 codes back coalesced.
 //
 // BOUND: both interval outputs in one launch (lower first, then upper) on the same staged pair of images, inverted
 // boxes collapsed to their midpoint while staging (reference: core/cuda/bound_inf_dist_cuda.cu:63).
@@ -36,17 +36,6 @@ struct ImageRowBlocks {
     float inv_pitch, inv_ow;
 };
 
-// Value of lane SUB of every group of eight lanes, in all lanes of the group, without the LDS crossbar: the quad that
-// holds the lane spreads it with a quad permutation, the other quad takes it from there through the mirror of the
-// eight lanes.
-template <int SUB>
-__device__ __forceinline__ int group_bcast(int v, int lane) {
-    constexpr int q = SUB & 3, ctrl = q | (q << 2) | (q << 4) | (q << 6);  // quad_perm [q, q, q, q]
-    const int own = __builtin_amdgcn_update_dpp(0, v, ctrl, 0xf, 0xf, true);
-    const int other = __builtin_amdgcn_update_dpp(0, own, 0x141, 0xf, 0xf, true);  // row_half_mirror
-    return ((lane >> 2) & 1) == (SUB >> 2) ? own : other;
-}
-
 template <bool BOUND, int KT>
 __global__ __launch_bounds__(1024) void rescan_image_kernel(const float* __restrict__ x, const float* __restrict__ x2,
                                                             const float* __restrict__ w, const float* __restrict__ out1,
@@ -55,7 +44,7 @@ __global__ __launch_bounds__(1024) void rescan_image_kernel(const float* __restr
                                                             const ImageRowBlocks rg, int w_vec) {
     extern __shared__ float lds[];
     constexpr uint32_t kNoKey = 0xffffffffu;
-    static_assert(KT == 16 || KT == 32, "eight lanes of four k cover a tile");
+    static_assert(KT == 16 || KT == 32, "four lanes of four k cover a tile in one or two steps");
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), nwave = (int)blockDim.x >> 6;
     unsigned id = blockIdx.x;
@@ -143,56 +132,59 @@ __global__ __launch_bounds__(1024) void rescan_image_kernel(const float* __restr
                 if (t < 0 || t >= rg.nt) t = -1;
             }
             const float* __restrict__ wrow = w + w_off(s, g, n, 0);
-            const int quad = (lane & 7) * 4;
             uint32_t mine = kNoKey;  // the result of the output this lane read
             auto step = [&](auto sub_c) __attribute__((always_inline)) {
                 constexpr int sub = decltype(sub_c)::value;
-                const int tt = group_bcast<sub>(t, lane), po = group_bcast<sub>(poff, lane);
-                const float target = __int_as_float(group_bcast<sub>(__float_as_int(val), lane));
+                constexpr int ctrl = sub | (sub << 2) | (sub << 4) | (sub << 6);  // quad_perm [sub, sub, sub, sub]
+                const int tt = __builtin_amdgcn_update_dpp(0, t, ctrl, 0xf, 0xf, true);
+                const int po = __builtin_amdgcn_update_dpp(0, poff, ctrl, 0xf, 0xf, true);
+                const float target = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(val), ctrl, 0xf, 0xf, true));
                 uint32_t key = kNoKey;
-                const int k = tt * KT + quad;
-                if (tt >= 0 && quad < KT && k < K) {
-                    float wv[4];
-                    if (w_vec) {
-                        const float4 w4 = *reinterpret_cast<const float4*>(wrow + k);
-                        wv[0] = w4.x; wv[1] = w4.y; wv[2] = w4.z; wv[3] = w4.w;
-                    } else {
+                if (tt >= 0) {
 #pragma unroll
-                        for (int j = 0; j < 4; j++) wv[j] = k + j < K ? wrow[k + j] : 0.f;
-                    }
-                    const int4 tp4 = *reinterpret_cast<const int4*>(tab + k);  // (k is a multiple of four)
-                    const int tp[4] = {tp4.x, tp4.y, tp4.z, tp4.w};
-                    float xa[4], xb[4];  // the reads leave together
+                    for (int h = KT / 16 - 1; h >= 0; h--) {  // descending: the lowest matching k is kept
+                        const int k = tt * KT + (lane & 3) * 4 + 16 * h;
+                        if (k < K) {
+                            float wv[4];
+                            if (w_vec) {
+                                const float4 w4 = *reinterpret_cast<const float4*>(wrow + k);
+                                wv[0] = w4.x; wv[1] = w4.y; wv[2] = w4.z; wv[3] = w4.w;
+                            } else {
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        xa[j] = xs[tp[j] + po];
-                        xb[j] = BOUND ? xs[cg * E + tp[j] + po] : 0.f;
-                    }
+                                for (int j = 0; j < 4; j++) wv[j] = k + j < K ? wrow[k + j] : 0.f;
+                            }
+                            const int4 tp4 = *reinterpret_cast<const int4*>(tab + k);  // (k is a multiple of four)
+                            const int tp[4] = {tp4.x, tp4.y, tp4.z, tp4.w};
+                            float xa[4], xb[4];  // the reads leave together
 #pragma unroll
-                    for (int j = 3; j >= 0; j--) {  // descending: the lowest matching k is kept
-                        bool hit, neg;
-                        if constexpr (!BOUND) {
-                            const float d = xa[j] - wv[j];
-                            hit = fabsf(d) == target;
-                            neg = !(d >= 0);
-                        } else {
-                            const float t1 = wv[j] - xa[j], t2 = xb[j] - wv[j];
-                            hit = (lower ? fminf(t1, t2) : fmaxf(t1, t2)) == target;
-                            neg = !(t1 <= t2);
+                            for (int j = 0; j < 4; j++) {
+                                xa[j] = xs[tp[j] + po];
+                                xb[j] = BOUND ? xs[cg * E + tp[j] + po] : 0.f;
+                            }
+#pragma unroll
+                            for (int j = 3; j >= 0; j--) {
+                                bool hit, neg;
+                                if constexpr (!BOUND) {
+                                    const float d = xa[j] - wv[j];
+                                    hit = fabsf(d) == target;
+                                    neg = !(d >= 0);
+                                } else {
+                                    const float t1 = wv[j] - xa[j], t2 = xb[j] - wv[j];
+                                    hit = (lower ? fminf(t1, t2) : fmaxf(t1, t2)) == target;
+                                    neg = !(t1 <= t2);
+                                }
+                                if (hit && k + j < K) key = ((uint32_t)(k + j) << 1) | (neg ? 1u : 0u);
+                            }
                         }
-                        if (hit && k + j < K) key = ((uint32_t)(k + j) << 1) | (neg ? 1u : 0u);
                     }
                 }
-                // lowest key of the eight lanes that share the output (all lanes of the wave are here)
+                // lowest key of the four lanes that share the output (all lanes of the wave are here)
                 key = min(key, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)key, 0xB1, 0xf, 0xf, true));   // quad_perm [1,0,3,2]
                 key = min(key, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)key, 0x4E, 0xf, 0xf, true));   // quad_perm [2,3,0,1]
-                key = min(key, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)key, 0x141, 0xf, 0xf, true));  // row_half_mirror
-                if ((lane & 7) == sub) mine = key;
+                if ((lane & 3) == sub) mine = key;
             };
             step(std::integral_constant<int, 0>{}); step(std::integral_constant<int, 1>{});
             step(std::integral_constant<int, 2>{}); step(std::integral_constant<int, 3>{});
-            step(std::integral_constant<int, 4>{}); step(std::integral_constant<int, 5>{});
-            step(std::integral_constant<int, 6>{}); step(std::integral_constant<int, 7>{});
             if (live) {
                 uint32_t code = kDefault;
                 if (t >= 0 && mine != kNoKey) code = (mine >> 1) | ((mine & 1u) ? kSignBit : 0u);
