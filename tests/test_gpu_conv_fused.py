@@ -74,7 +74,7 @@ TRAIN_CASES = CASES + [
                                                    # sorted second pass gathers the patches instead
     (2, 300, 6, 6, 7, 1, 3, 1, 1, 1),              # 300 channels: one workgroup of 1024 threads per compute unit
     (1, 3, 100, 120, 6, 1, 5, 1, 2, 2),            # a larger plane, window 5, stride 2: several row blocks per sample
-    (2, 6, 40, 24, 9, 2, (3, 2), (2, 1), (2, 0), (1, 2)),  # dilated rows, strided columns, two groups
+    (2, 6, 40, 24, 10, 2, (3, 2), (2, 1), (2, 0), (1, 2)),  # dilated rows, strided columns, two groups
 ]
 
 
