@@ -244,6 +244,15 @@ def other_workloads(torch, _C, xd, wd, gd):
             conv(cd, cd - 8 / 255, cd + 8 / 255)
 
     res["conv3x3_128to128_b128_32x32_pinf_eval_with_ibp"] = tm(conv_ibp)
+    # the layer's forward alone with arg-max codes (first pass + second pass), and its training step at p = 8
+    cw = conv.weight.detach()
+    cy = torch.empty(128, 128, 1024, device=dev)
+    cpos = torch.empty(128, 128, 1024, device=dev, dtype=torch.int32)
+    res["conv3x3_128to128_b128_32x32_pinf_forward_with_codes"] = tm(
+        lambda: _C.conv_inf_dist_forward(cd, cw, cy, cpos, 1, 3, 1, 1, 1))
+    conv.train()
+    conv.p = 8.0
+    res["conv3x3_128to128_b128_32x32_p8_fwd_bwd"] = tm(conv_step)
     return res
 
 
