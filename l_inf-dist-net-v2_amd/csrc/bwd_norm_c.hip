@@ -44,7 +44,6 @@ __global__ __launch_bounds__(256) void bwd_gx_fixup_kernel(const float* __restri
     const Geom& s = P.s;
     // (1024 elements of a block per workgroup)
     const int nchunk = (rows_per_wg * kBwdSlab + 1023) / 1024;
-    const long sr = blockIdx.x / (unsigned)nchunk, b0 = sr * P.ncc, b1 = b0 + P.ncc;
     const int e0 = (int)(blockIdx.x % (unsigned)nchunk) * 1024;
     auto begin = [&](long g) { return g * P.total / nwg; };
     auto owner = [&](long u) {  // the workgroup whose range holds unit u
@@ -54,8 +53,15 @@ __global__ __launch_bounds__(256) void bwd_gx_fixup_kernel(const float* __restri
         while (g + 1 < nwg && begin(g + 1) <= u) g++;
         return g;
     };
+    // The grid runs over the boundaries between workgroups, not over all blocks: only a block with a boundary inside
+    // is split (with few output columns the blocks are short and almost all of them whole).  A block that holds
+    // several boundaries belongs to the first of them.
+    const long first = blockIdx.x / (unsigned)nchunk;  // the boundary between workgroups `first` and `first` + 1
+    const long ub = begin(first + 1);
+    if (ub % P.ncc == 0) return;                       // it falls between two blocks
+    const long sr = ub / P.ncc, b0 = sr * P.ncc, b1 = b0 + P.ncc;
     const long g_lo = owner(b0), g_hi = owner(b1 - 1);
-    if (g_lo == g_hi) return;
+    if (g_lo != first || g_lo == g_hi) return;
     const int rc = (int)(sr % P.nrc);
     const int gs = (int)(sr / P.nrc);
     const int grp = gs / P.nslab, ci0 = (gs - grp * P.nslab) * kBwdSlab;
@@ -470,9 +476,11 @@ int launch_norm_backward(const float* gout, const float* x, const float* w, cons
         }
     }
     if (!rc && part != nullptr) {
-        const long nblk = (long)s.G * P.nslab * P.nrc * ((rows_per_wg * kBwdSlab + 1023) / 1024);
-        hipLaunchKernelGGL(bwd_gx_fixup_kernel, dim3((unsigned)nblk), dim3(256), 0, st, part, gx_k, P, grid, rows_per_wg);
-        if (hip_failed(hipGetLastError())) rc = 4;
+        const long nblk = (long)(grid - 1) * ((rows_per_wg * kBwdSlab + 1023) / 1024);
+        if (nblk > 0) {
+            hipLaunchKernelGGL(bwd_gx_fixup_kernel, dim3((unsigned)nblk), dim3(256), 0, st, part, gx_k, P, grid, rows_per_wg);
+            if (hip_failed(hipGetLastError())) rc = 4;
+        }
     }
     if (part != nullptr && hip_failed(scratch_free(part, st)) && !rc) rc = 4;
     if (!rc && cv != nullptr) rc = launch_fold_rows(gx_k, *cv, gx, st);
