@@ -76,8 +76,10 @@ __global__ __launch_bounds__(256) void fold_kernel(const float* __restrict__ gou
 __global__ __launch_bounds__(256) void patch_rows_kernel(const float* __restrict__ x, float* __restrict__ out,
                                                          const UnfoldGeom u, int CC, int ncb, int vec4, float inv_w,
                                                          float inv_ccw, float inv_taps, float inv_kw) {
-    extern __shared__ float strip[];  // [kh][CC][WP], WP = W | 1: neighbouring channels in different banks
+    extern __shared__ float strip[];  // [kh][CC][WP], WP = W | 1: neighbouring channels in different banks; then the
+                                      // offsets of the block's CC * taps values inside the strip
     const int WP = u.W | 1;
+    int* __restrict__ tapoff = reinterpret_cast<int*>(strip + u.kh * CC * WP);
     unsigned id = blockIdx.x;
     const int cb = (int)(id % (unsigned)ncb);
     id /= (unsigned)ncb;
@@ -93,14 +95,19 @@ __global__ __launch_bounds__(256) void patch_rows_kernel(const float* __restrict
         strip[(i * CC + cl) * WP + wc] =
             (cl < ncl && (unsigned)h < (unsigned)u.H) ? x[(((long)b * u.C + c0 + cl) * u.H + h) * u.W + wc] : 0.f;
     }
+    // value kk of a run: strip offset of its row start and its column shift, worked out once per workgroup
+    for (int kk = threadIdx.x; kk < CC * taps; kk += 256) {
+        const int cl = small_div(kk, taps, inv_taps), tap = kk - cl * taps;
+        const int i = small_div(tap, u.kw, inv_kw), j = tap - i * u.kw;
+        tapoff[kk] = ((i * CC + cl) * WP << 8) | (j * u.dw);  // (the launcher keeps the shift below 256)
+    }
     __syncthreads();
     const int run = ncl * taps;  // contiguous floats per output position
     float* __restrict__ dst = out + ((long)b * L + (long)oh * u.OW) * K + (long)c0 * taps;
     auto value = [&](int ow, int kk) {
-        const int cl = small_div(kk, taps, inv_taps), tap = kk - cl * taps;
-        const int i = small_div(tap, u.kw, inv_kw), j = tap - i * u.kw;
-        const int wc = ow * u.sw - u.pw + j * u.dw;
-        return (unsigned)wc < (unsigned)u.W ? strip[(i * CC + cl) * WP + wc] : 0.f;
+        const int t = tapoff[kk];
+        const int wc = ow * u.sw - u.pw + (t & 0xff);
+        return (unsigned)wc < (unsigned)u.W ? strip[(t >> 8) + wc] : 0.f;
     };
     if (vec4) {  // run and K are multiples of four and out is 16-byte aligned: one store per four values
         const int run4 = run >> 2;
@@ -187,6 +194,7 @@ bool patch_rows_applies(const UnfoldGeom& u) {
     CC = CC > u.C ? u.C : CC;
     if (CC >= 4 && CC < u.C) CC &= ~3;
     if (CC < 1 || (long)u.kh * CC * u.W >= (1L << 22) || (long)u.OW * CC * taps >= (1L << 22)) return false;
+    if ((long)(u.kw - 1) * u.dw >= 256 || (long)CC * taps > 8192) return false;  // packed tap offsets, 32 KB of them at most
     return (long)u.B * u.OH * ((u.C + CC - 1) / CC) < (1L << 31);
 }
 
@@ -197,12 +205,14 @@ int launch_patch_rows(const float* x, const UnfoldGeom& u, float* out, hipStream
     CC = CC > u.C ? u.C : CC;
     if (CC >= 4 && CC < u.C) CC &= ~3;  // whole quads of channels: every run of a workgroup then allows 16-byte stores
     if (CC < 1 || (long)u.kh * CC * u.W >= (1L << 22) || (long)u.OW * CC * taps >= (1L << 22)) return -1;
+    if ((long)(u.kw - 1) * u.dw >= 256 || (long)CC * taps > 8192) return -1;
     const int ncb = (u.C + CC - 1) / CC;
     const long blocks = (long)u.B * u.OH * ncb;
     if (blocks >= (1L << 31)) return -1;
     // 16-byte stores need every run of a workgroup to start and end on a multiple of four floats
     const int vec4 = (CC * taps) % 4 == 0 && (u.C * taps) % 4 == 0 && (uintptr_t)out % 16 == 0;
-    hipLaunchKernelGGL(patch_rows_kernel, dim3((unsigned)blocks), dim3(256), (size_t)u.kh * CC * (u.W | 1) * sizeof(float), st, x,
+    hipLaunchKernelGGL(patch_rows_kernel, dim3((unsigned)blocks), dim3(256),
+                       ((size_t)u.kh * CC * (u.W | 1) + (size_t)CC * taps) * sizeof(float), st, x,
                        out, u, CC, ncb, vec4, 1.0f / (float)u.W, 1.0f / (float)(CC * u.W), 1.0f / (float)taps,
                        1.0f / (float)u.kw);
     return hip_failed(hipGetLastError()) ? 4 : 0;
