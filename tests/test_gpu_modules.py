@@ -200,3 +200,21 @@ def test_hybrid_model_margins_are_sound_and_trainable():
     margin.clamp(min=0).sum().backward()
     grads = [p.grad for n, p in model.named_parameters() if "fc_dist" in n and p.grad is not None]
     assert grads and all(torch.isfinite(g).all() for g in grads) and any(float(g.abs().sum()) > 0 for g in grads)
+
+
+def test_empty_batch_on_the_device():
+    """An empty batch returns empty outputs and zero gradients without touching the library (the reference's launches
+    over no rows do the same, core/cuda/norm_dist_cuda.cu:515-520, 602-604)."""
+    from core.norm_dist import norm_dist, bound_inf_dist, conv_norm_dist
+    w = torch.randn(6, 8, device="cuda", requires_grad=True)
+    x = torch.zeros(0, 8, 3, device="cuda", requires_grad=True)
+    for p in (8.0, float("inf")):
+        w.grad = None
+        y = norm_dist(x, w, p)
+        assert y.shape == (0, 6, 3) and y.is_cuda
+        y.sum().backward()
+        assert torch.equal(w.grad, torch.zeros_like(w))
+    lo, up = bound_inf_dist(x.detach(), x.detach(), w.detach())
+    assert lo.shape == up.shape == (0, 6, 3)
+    wc = torch.randn(5, 36, device="cuda")
+    assert conv_norm_dist(torch.zeros(0, 4, 7, 7, device="cuda"), wc, float("inf"), 3, 1, 1, 2).shape == (0, 5, 16)
