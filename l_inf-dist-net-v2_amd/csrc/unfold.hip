@@ -180,9 +180,108 @@ __global__ __launch_bounds__(256) void fold_rows_kernel(const float* __restrict_
     }
 }
 
+// The same sums from fewer, wider loads.  The kw taps of one window row lie side by side in memory, so a thread first
+// adds, for one position and one channel, the taps of those window rows that reach image row h (4 * kw bytes per
+// load, and which window rows reach h is the same for the whole workgroup), and leaves its kw sums in LDS; a pixel is
+// then the sum of one tap from each of kw neighbouring positions.  KW: the window's width, 0 = any (one tap per
+// load).  Fixed order of additions: reproducible.
+template <int KW, bool UNIT>
+__global__ __launch_bounds__(256) void fold_rows_taps_kernel(const float* __restrict__ g, float* __restrict__ gx,
+                                                             const UnfoldGeom u, const int now, const int pitch) {
+    extern __shared__ float part[];  // [64 channels][pitch >= now * kw]
+    const int nwb = (u.W + 31) / 32, ncb = (u.C + 63) / 64;
+    unsigned id = blockIdx.x;
+    const int wb = (int)(id % (unsigned)nwb);
+    id /= (unsigned)nwb;
+    const int cb = (int)(id % (unsigned)ncb);
+    id /= (unsigned)ncb;
+    const int h = (int)(id % (unsigned)u.H), b = (int)(id / (unsigned)u.H);
+    const int kw = KW ? KW : u.kw, taps = u.kh * kw, L = u.OH * u.OW;
+    const long K = (long)u.C * taps;
+    // first position whose window reaches the block's first pixel column
+    const int lo = wb * 32 + u.pw - (kw - 1) * u.dw;
+    const int ow0 = lo <= 0 ? 0 : (UNIT ? lo : (lo + u.sw - 1) / u.sw);
+    const int cl = threadIdx.x & 63, c = cb * 64 + cl;
+    if (c < u.C) {
+        const float* __restrict__ gb = g + (long)b * L * K + (long)c * taps;
+        for (int ol = threadIdx.x >> 6; ol < now; ol += 4) {
+            const int ow = ow0 + ol;
+            if (ow >= u.OW) break;
+            float p[KW ? KW : 1];
+#pragma unroll
+            for (int j = 0; j < (KW ? KW : 1); j++) p[j] = 0.f;
+            if (KW) {
+                for (int i = 0; i < u.kh; i++) {
+                    const int hn = h + u.ph - i * u.dh;
+                    int oh = hn;
+                    if (!UNIT) {
+                        if (hn < 0 || hn % u.sh != 0) continue;
+                        oh = hn / u.sh;
+                    }
+                    if ((unsigned)oh >= (unsigned)u.OH) continue;
+                    const float* __restrict__ src = gb + (long)(oh * u.OW + ow) * K + i * KW;
+#pragma unroll
+                    for (int j = 0; j < KW; j++) p[j] += src[j];
+                }
+#pragma unroll
+                for (int j = 0; j < KW; j++) part[cl * pitch + ol * KW + j] = p[j];
+            } else {
+                for (int j = 0; j < kw; j++) {
+                    float acc = 0.f;
+                    for (int i = 0; i < u.kh; i++) {
+                        const int hn = h + u.ph - i * u.dh;
+                        int oh = hn;
+                        if (!UNIT) {
+                            if (hn < 0 || hn % u.sh != 0) continue;
+                            oh = hn / u.sh;
+                        }
+                        if ((unsigned)oh >= (unsigned)u.OH) continue;
+                        acc += gb[(long)(oh * u.OW + ow) * K + i * kw + j];
+                    }
+                    part[cl * pitch + ol * kw + j] = acc;
+                }
+            }
+        }
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < 64 * 32; idx += 256) {
+        const int cc = idx >> 5, w = wb * 32 + (idx & 31);
+        const int c2 = cb * 64 + cc;
+        if (c2 >= u.C || w >= u.W) continue;
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < (KW ? KW : kw); j++) {
+            const int wn = w + u.pw - j * u.dw;
+            int ow = wn;
+            if (!UNIT) {
+                if (wn < 0 || wn % u.sw != 0) continue;
+                ow = wn / u.sw;
+            }
+            if ((unsigned)ow >= (unsigned)u.OW) continue;
+            acc += part[cc * pitch + (ow - ow0) * kw + j];
+        }
+        gx[(((long)b * u.C + c2) * u.H + h) * u.W + w] = acc;
+    }
+}
+
 int launch_fold_rows(const float* g, const UnfoldGeom& u, float* gx, hipStream_t st) {
     const long blocks = (long)u.B * u.H * ((u.C + 63) / 64) * ((u.W + 31) / 32);
     if (blocks >= (1L << 31)) return 2;
+    // positions whose windows reach a block of 32 pixel columns
+    const long now = (31 + (long)(u.kw - 1) * u.dw) / u.sw + 2, pitch = (now * u.kw) | 1;
+    if (u.kw >= 2 && 64 * pitch * sizeof(float) <= 64 * 1024) {
+        const size_t lds = 64 * (size_t)pitch * sizeof(float);
+        const bool unit = u.sh == 1 && u.sw == 1;
+#define NDIST_FOLD_TAPS(KW, UNIT) \
+    hipLaunchKernelGGL((fold_rows_taps_kernel<KW, UNIT>), dim3((unsigned)blocks), dim3(256), lds, st, g, gx, u, (int)now, \
+                       (int)pitch)
+        if (u.kw == 3 && unit) NDIST_FOLD_TAPS(3, true);
+        else if (u.kw == 3) NDIST_FOLD_TAPS(3, false);
+        else if (unit) NDIST_FOLD_TAPS(0, true);
+        else NDIST_FOLD_TAPS(0, false);
+#undef NDIST_FOLD_TAPS
+        return hip_failed(hipGetLastError()) ? 4 : 0;
+    }
     if (u.sh == 1 && u.sw == 1) hipLaunchKernelGGL(fold_rows_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, st, g, gx, u);
     else hipLaunchKernelGGL(fold_rows_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, st, g, gx, u);
     return hip_failed(hipGetLastError()) ? 4 : 0;

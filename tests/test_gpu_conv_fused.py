@@ -23,6 +23,8 @@ CASES = [  # B, C, H, W, CO, G, kernel, dilation, padding, stride
     (1, 256, 8, 8, 32, 1, 3, 1, 1, 1),             # one output tile, k = 2304: k range split over workgroups
     (2, 40, 16, 16, 200, 1, 3, 1, 1, 1),           # ragged column tiles, k = 360 not a multiple of the stage
     (1, 3, 5, 5, 3, 1, 3, 1, 2, 1),                # padding wider than one tap: whole patches of zeros at corners
+    (1, 3, 4, 70, 4, 1, 3, 1, 1, 1),               # wider than one block of 32 pixel columns (the adjoint's halo)
+    (1, 2, 5, 75, 3, 1, (2, 5), (1, 2), (0, 3), (1, 2)),  # the same with a wide dilated window and a stride
 ]
 
 
