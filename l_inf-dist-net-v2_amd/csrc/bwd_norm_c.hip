@@ -303,10 +303,15 @@ static BwdPlan plan_backward(const Geom& s, float p) {
         // variant of the large exponents costs per chunk rather than per row (1, 0.75, 0.6: it spends its time on
         // the weights and factors of a unit, not on the rows); which variant will run is not known here, so the
         // large exponents use the mean of the two cost vectors.
+        // With few output columns the rows change every few units, and a workgroup's waves then all wait for the new
+        // rows together: two 8-wave workgroups per compute unit cover each other's waits, one of 16 waves cannot
+        // (3 x 3 conv, 128 channels: 3 - 6 % faster at 64 ... 512 output columns, 0 - 7 % slower at 1024).
         constexpr double kChunkCost[2][3] = {{1.0, 0.505, 0.28}, {1.0, 0.63, 0.44}};
+        const bool few_columns = ceil_div(s.COg, kBwdCoUnit) <= 32;
         double best = 0.0;
         for (int c = 0; c < 3; c++) {
-            const double cost = kChunkCost[pl.want_adaptive ? 1 : 0][c] * ceil_div(s.M, kBwdCfgRows[c] * kBwdCfgWaves[c]);
+            double cost = kChunkCost[pl.want_adaptive ? 1 : 0][c] * ceil_div(s.M, kBwdCfgRows[c] * kBwdCfgWaves[c]);
+            if (c == 1 && few_columns && !pl.want_adaptive) cost *= 0.94;
             if (c == 0 || cost < best) { best = cost; pl.cfg = c; }
         }
         if (s.M <= 64) pl.cfg = 4;  // one 64-row chunk (0.33 ms at 5120 x 5120 against 0.51 for a 128-row chunk)
