@@ -61,7 +61,18 @@ struct BwdParams {
     // in) and bwd_gx_fixup_kernel adds the shares in workgroup order.  nullptr: global atomic adds into a zeroed
     // grad_input (sums in arrival order).
     float* part;
+    // Rows that are the patches of images (convolutional layer): when `image` is set, row m = (sample, output position)
+    // is not read from memory laid out [M][CI] but gathered from the images [B][C][H][W] of geometry `cv`, zeros
+    // outside the image, column ci of group g being tap (g * CIg + ci) of the unfolded problem.  Main kernel only.
+    // The description lives in device memory, not among the kernel's arguments: its fields are then fetched where the
+    // rows change and nowhere else (as arguments they cost the main loop scalar registers it does not have).
+    const struct BwdImage* image;
 };
+struct BwdImage {
+    const float* img;
+    UnfoldGeom cv;
+};
+static_assert(sizeof(BwdImage) == 64 && offsetof(BwdImage, cv) == 8, "read below as sixteen words");
 
 typedef float f16v __attribute__((ext_vector_type(16)));
 // 16 consecutive factors through the scalar data cache: a load from the constant address space with a wave-uniform
@@ -416,14 +427,50 @@ __global__ __launch_bounds__(64 * NW, 4) void bwd_fused_kernel(const float* __re
             xci = cur.ci0 + lane;
             x_ok = xci < s.CIg;
             xr0 = (cur.rc * NW + wave) * BT;
+            if (P.image != nullptr) {
+                typedef int i16v __attribute__((ext_vector_type(16)));
+                typedef const i16v __attribute__((address_space(4))) * cptr;
+                const i16v raw = *reinterpret_cast<cptr>(reinterpret_cast<uintptr_t>(P.image));  // one scalar load
+                const float* __restrict__ img = reinterpret_cast<const float*>(
+                    ((unsigned long long)(unsigned)raw[1] << 32) | (unsigned long long)(unsigned)raw[0]);
+                UnfoldGeom cv;
+                cv.B = raw[2], cv.C = raw[3], cv.H = raw[4], cv.W = raw[5], cv.kh = raw[6], cv.kw = raw[7];
+                cv.dh = raw[8], cv.dw = raw[9], cv.ph = raw[10], cv.pw = raw[11], cv.sh = raw[12], cv.sw = raw[13];
+                cv.OH = raw[14], cv.OW = raw[15];
+                // the lane's tap: channel and pixel offset inside the window (once per change of rows)
+                const int col = xg * s.CIg + xci, taps = cv.kh * cv.kw;
+                const int c = col / taps, tap = col - c * taps;
+                const int ti = tap / cv.kw, tj = tap - ti * cv.kw;
+                const int hi = ti * cv.dh - cv.ph, wj = tj * cv.dw - cv.pw;
+                const long lane_off = ((long)c * cv.H + hi) * cv.W + wj;
+                // the wave's first row: sample and output position, stepped from row to row
+                const int L = cv.OH * cv.OW;
+                int b = xr0 / L, oh = (xr0 - b * L) / cv.OW, ow = xr0 - b * L - oh * cv.OW;
 #pragma unroll
-            for (int i = 0; i < BT; i++) {
-                const int m = xr0 + i;
-                gxa[i] = 0.f;
-                xv[i] = 0.f;
-                if (x_ok && m < s.M) {
-                    const int b = m / s.HW, hw = m - b * s.HW;
-                    xv[i] = X[x_off(s, b, xg, xci, hw)];
+                for (int i = 0; i < BT; i++) {
+                    gxa[i] = 0.f;
+                    xv[i] = 0.f;
+                    const int h0 = oh * cv.sh, w0 = ow * cv.sw;
+                    if (x_ok && xr0 + i < s.M && (unsigned)(h0 + hi) < (unsigned)cv.H && (unsigned)(w0 + wj) < (unsigned)cv.W)
+                        xv[i] = img[((long)b * cv.C * cv.H + h0) * cv.W + w0 + lane_off];
+                    if (++ow == cv.OW) {
+                        ow = 0;
+                        if (++oh == cv.OH) {
+                            oh = 0;
+                            b++;
+                        }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < BT; i++) {
+                    const int m = xr0 + i;
+                    gxa[i] = 0.f;
+                    xv[i] = 0.f;
+                    if (x_ok && m < s.M) {
+                        const int b = m / s.HW, hw = m - b * s.HW;
+                        xv[i] = X[x_off(s, b, xg, xci, hw)];
+                    }
                 }
             }
             if constexpr (IP == -4) {

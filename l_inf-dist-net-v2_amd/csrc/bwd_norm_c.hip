@@ -323,6 +323,18 @@ static BwdPlan plan_backward(const Geom& s, float p) {
     return pl;
 }
 
+// the description of the images goes to device memory through a kernel, so that it is part of a captured graph
+__global__ void bwd_image_kernel(const BwdImage v, BwdImage* __restrict__ dst) {
+    if (threadIdx.x == 0) *dst = v;
+}
+
+// NORM_DIST_BWD_GATHER=0: the patches of a conv layer are always written out as rows first (the path of the
+// skipping variants and of small batches); read at every call
+static bool bwd_gather_enabled() {
+    const char* e = getenv("NORM_DIST_BWD_GATHER");
+    return e == nullptr || e[0] != '0';
+}
+
 size_t norm_backward_scratch_bytes(const Geom& s, float p) {
     const BwdPlan pl = plan_backward(s, p);
     const size_t mpad = (size_t)ceil_div(s.M, pl.rows_per_wg) * pl.rows_per_wg;
@@ -382,7 +394,28 @@ int launch_norm_backward(const float* gout, const float* x, const float* w, cons
     bool transposed = cv != nullptr || (s.HW >= kBwdTransposeMinHW && s.B <= 65535);
     float* xT = nullptr;  // [M][CI] copy of x, followed by the [M][CI] gradient (and the unfolded buffer)
     float* unfolded = nullptr;
-    if (!rc && transposed) {
+    // The main kernel gathers the patches from the images itself (BwdParams::img): no copy of x in the row layout,
+    // only the gradient rows.  (The probes of the skipping variants and the small-batch kernel read rows.)
+    const bool gather = cv != nullptr && !adaptive && cfg != 3 && bwd_gather_enabled();
+    if (!rc && gather) {
+        const hipError_t e = scratch_alloc((void**)&xT, (size_t)nx * sizeof(float), st);
+        if (e != hipSuccess) {
+            (void)scratch_free(aT, st);
+            return hip_status(e);
+        }
+        P.s.B = s.M;
+        P.s.HW = 1;
+        BwdImage* image = nullptr;
+        const hipError_t e2 = scratch_alloc((void**)&image, sizeof(BwdImage), st);
+        if (e2 != hipSuccess) {
+            (void)scratch_free(xT, st);
+            (void)scratch_free(aT, st);
+            return hip_status(e2);
+        }
+        hipLaunchKernelGGL(bwd_image_kernel, dim3(1), dim3(64), 0, st, BwdImage{x, *cv}, image);
+        if (hip_failed(hipGetLastError())) rc = 4;
+        P.image = image;
+    } else if (!rc && transposed) {
         const bool via_unfold = cv != nullptr && !patch_rows_applies(*cv);  // needs the third buffer
         const hipError_t e = scratch_alloc((void**)&xT, (via_unfold ? 3 : 2) * (size_t)nx * sizeof(float), st);
         if (e != hipSuccess && cv != nullptr) {  // on images there is no other path
@@ -412,7 +445,7 @@ int launch_norm_backward(const float* gout, const float* x, const float* w, cons
                 rc = launch_norm_probe(xT, w, P.s, exp2f(-40.0f / q), reinterpret_cast<int*>(aux), st);
         }
     }
-    float* gx_k = transposed ? xT + nx : gx;
+    float* gx_k = gather ? xT : (transposed ? xT + nx : gx);
     // Reproducible grad_input: shares of the blocks that two workgroups split go through a buffer and are added in a
     // fixed order (see BwdParams::part).  Not for the small-batch kernel, not where several kernel variants are
     // queued (their grids may differ), not from the fixed scratch array (64 MB at the headline shape): those add
@@ -490,6 +523,7 @@ int launch_norm_backward(const float* gout, const float* x, const float* w, cons
     if (part != nullptr && hip_failed(scratch_free(part, st)) && !rc) rc = 4;
     if (!rc && cv != nullptr) rc = launch_fold_rows(gx_k, *cv, gx, st);
     else if (!rc && transposed) rc = transpose_batched(gx_k, gx, s.B, s.HW, s.CIg * s.G, st);
+    if (P.image != nullptr && hip_failed(scratch_free(const_cast<BwdImage*>(P.image), st)) && !rc) rc = 4;
     if (xT != nullptr && hip_failed(scratch_free(xT, st)) && !rc) rc = 4;
     if (aux != nullptr && hip_failed(scratch_free(aux, st)) && !rc) rc = 4;
     if (hip_failed(scratch_free(aT, st)) && !rc) rc = 4;

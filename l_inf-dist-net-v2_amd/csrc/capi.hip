@@ -504,7 +504,8 @@ static int conv_norm_backward(const float* grad_output, const float* input, cons
     if (int rc = make_conv_geom(B, C, H, W, CO, G, kernel_h, kernel_w, dilation_h, dilation_w, padding_h, padding_w,
                                 stride_h, stride_w, &u, &s))
         return rc;
-    // The backward's kernel reads the patches as rows and writes gradient rows: two buffers of the unfolded size
+    // The backward's kernel writes gradient rows and, where it does not gather the patches from the images itself
+    // (term-skipping variants, tiny batches), reads the patches as rows: one or two buffers of the unfolded size
     // (B x C kh kw x OH OW floats each, 604 MB at 128 x 128 x 32 x 32 with 3 x 3 windows).  Batches whose buffers
     // would exceed 256 MiB each are processed in parts of whole samples, grad_weight accumulating
     // over the parts: the scratch stays bounded whatever the batch, at a small cost in time (the parts are long enough

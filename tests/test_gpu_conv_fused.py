@@ -290,6 +290,34 @@ def test_conv_norm_dist_backward_in_parts_of_the_batch(p, G, stride, monkeypatch
     assert_close(only_x.cpu().numpy(), ex_img, tol=tol_x, what="input-only entry point in parts p=%g" % p)
 
 
+@pytest.mark.parametrize("p", [2.0, 8.0])
+@pytest.mark.parametrize("B,C,H,W,CO,G,k,d,p_,s", [CASES[1], CASES[2], CASES[4], CASES[7], CASES[-1]])
+def test_conv_norm_dist_backward_from_patch_rows(B, C, H, W, CO, G, k, d, p_, s, p, monkeypatch):
+    """The finite-p backward on images gathers the patches inside its main kernel; NORM_DIST_BWD_GATHER=0 makes it
+    write them out as rows first (the route of the term-skipping variants and of batches of at most 32 positions):
+    the same rows, so the same gradients bit for bit, and within 1e-5 of the oracle."""
+    from core import _C
+    from util import backward_tolerances
+    x, w = _case(B * 59 + W, B, C, H, W, CO, G, k, d, p_, s)
+    patches = F.unfold(x, k, d, p_, s)
+    xd, wd = x.cuda(), w.cuda()
+    out = torch.empty(B, CO, patches.size(2), device="cuda")
+    _C.conv_norm_dist_forward(xd, wd, out, G, p, k, d, p_, s)
+    g = torch.randn(out.shape, generator=torch.Generator().manual_seed(5))
+    ex, ew = O.norm_dist_backward(g.numpy(), patches.numpy(), w.numpy(), out.cpu().numpy(), p, G)
+    ex_img = F.fold(torch.from_numpy(ex), (H, W), k, d, p_, s).numpy()
+    tol_x, tol_w = backward_tolerances(g.numpy(), patches.numpy(), w.numpy(), out.cpu().numpy(), p, G, ex, ew)
+    got = []
+    for mode in ("1", "0"):
+        monkeypatch.setenv("NORM_DIST_BWD_GATHER", mode)
+        gx, gw = torch.full_like(xd, float("nan")), torch.full_like(wd, float("nan"))
+        _C.conv_norm_dist_backward_input_weight(g.cuda(), xd, wd, out, gx, gw, G, p, k, d, p_, s)
+        assert_close(gx.cpu().numpy(), ex_img, tol=tol_x, what="grad_input, gather %s" % mode)
+        assert_close(gw.cpu().numpy(), ew, tol=tol_w, what="grad_weight, gather %s" % mode)
+        got.append((gx.cpu().numpy(), gw.cpu().numpy()))
+    np.testing.assert_array_equal(got[0][0], got[1][0])
+
+
 @pytest.mark.parametrize("B,C,H,W,CO,G,k,d,p,s", [CASES[2], CASES[6], CASES[7], CASES[9]])
 def test_conv_codes_with_the_sorted_second_pass(B, C, H, W, CO, G, k, d, p, s, monkeypatch):
     """The arg-max codes of the image entry points come from one of two second passes (staged image rows where they
