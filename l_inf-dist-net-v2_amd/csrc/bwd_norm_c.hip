@@ -335,6 +335,11 @@ static bool bwd_gather_enabled() {
     return e == nullptr || e[0] != '0';
 }
 
+bool norm_backward_gathers(const Geom& s, float p) {
+    const BwdPlan pl = plan_backward(s, p);
+    return !pl.want_adaptive && pl.cfg != 3 && bwd_gather_enabled();
+}
+
 size_t norm_backward_scratch_bytes(const Geom& s, float p) {
     const BwdPlan pl = plan_backward(s, p);
     const size_t mpad = (size_t)ceil_div(s.M, pl.rows_per_wg) * pl.rows_per_wg;
@@ -396,7 +401,7 @@ int launch_norm_backward(const float* gout, const float* x, const float* w, cons
     float* unfolded = nullptr;
     // The main kernel gathers the patches from the images itself (BwdParams::img): no copy of x in the row layout,
     // only the gradient rows.  (The probes of the skipping variants and the small-batch kernel read rows.)
-    const bool gather = cv != nullptr && !adaptive && cfg != 3 && bwd_gather_enabled();
+    const bool gather = cv != nullptr && !want_adaptive && cfg != 3 && bwd_gather_enabled();
     if (!rc && gather) {
         const hipError_t e = scratch_alloc((void**)&xT, (size_t)nx * sizeof(float), st);
         if (e != hipSuccess) {

@@ -511,10 +511,12 @@ static int conv_norm_backward(const float* grad_output, const float* input, cons
     // over the parts: the scratch stays bounded whatever the batch, at a small cost in time (the parts are long enough
     // to fill the device and grad_weight is added with atomics from the second row chunk on anyway: three parts of
     // 43 samples at that shape take 4 % longer than one piece).
+    // Where the kernel gathers, the one buffer may be twice as large: the same 512 MiB in all, in fewer parts.
     size_t budget = 256u << 20;
     if (const char* mb = getenv("NORM_DIST_CONV_PART_MB")) {  // tuning / test aid: budget per buffer in MiB
-        if (atol(mb) > 0) budget = (size_t)atol(mb) << 20;
+        if (atof(mb) > 0) budget = (size_t)(atof(mb) * 1048576.0);
     }
+    if (norm_backward_gathers(s, p)) budget *= 2;
     const size_t per_sample = (size_t)s.CIg * s.G * s.HW * sizeof(float);
     int part = (int)std::max<size_t>(1, budget / std::max<size_t>(1, per_sample));
     part = ceil_div(B, ceil_div(B, part));  // parts of equal size

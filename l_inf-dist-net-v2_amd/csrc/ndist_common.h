@@ -320,6 +320,9 @@ int launch_norm_backward(const float* gout, const float* x, const float* w, cons
 int fill_zero(float* p, long n, hipStream_t st);
 // bytes of scratch launch_norm_backward cannot do without (the factor array); everything else it asks for is optional
 size_t norm_backward_scratch_bytes(const Geom& s, float p);
+// whether the finite-p backward of a conv layer of this (unfolded) geometry gathers its patches from the images, i.e.
+// needs one buffer of the unfolded size instead of two
+bool norm_backward_gathers(const Geom& s, float p);
 // With a patch geometry the input gradients are images [B, C, H, W] (the adjoint of the patch extraction is applied
 // on the fly); the launcher returns -1 when the geometry does not fit its kernels and nothing was launched.
 int launch_inf_backward(const float* gout, const int32_t* pos, const Geom& s, float* gx, float* gw, hipStream_t st,
