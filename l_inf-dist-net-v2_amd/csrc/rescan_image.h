@@ -12,8 +12,8 @@
 // of 64 consecutive positions of one output channel with coalesced loads, hands them to its quads by quad
 // permutations (no trip through the LDS crossbar), and writes the 64 codes back coalesced.
 //
-// BOUND: both interval outputs in one launch (lower first, then upper) on the same staged pair of images, inverted
-// boxes collapsed to their midpoint while staging (reference: core/cuda/bound_inf_dist_cuda.cu:63).
+// BOUND: both interval outputs in one launch, and in one walk where they peak in the same tile, on the same staged
+// pair of images, inverted boxes collapsed to their midpoint while staging (reference: core/cuda/bound_inf_dist_cuda.cu:63).
 #pragma once
 #include "ndist_common.h"
 #include <algorithm>
@@ -109,86 +109,106 @@ __global__ __launch_bounds__(1024) void rescan_image_kernel(const float* __restr
     // ---- every output looks at its winning tile
     const int nmacro = (npos + 63) >> 6;  // blocks of 64 consecutive positions
     const int total = s.COg * nmacro;
+    // BOUND: the lower and the upper output of a box usually peak in the same tile (always, when the box has the same
+    // width everywhere): one walk over that tile then serves both; an upper output with a tile of its own gets a
+    // second walk.
 #pragma unroll 1
-    for (int side = 0; side < (BOUND ? 2 : 1); side++) {
-        const float* __restrict__ out = side == 0 ? out1 : out2;
-        int32_t* __restrict__ pos = side == 0 ? pos1 : pos2;
-        const bool lower = BOUND && side == 0;
-        const uint32_t kDefault = lower ? kNoGradId : 0u;
-#pragma unroll 1
-        for (int it = wave; it < total; it += nwave) {
-            const int n = it / nmacro, p = (it - n * nmacro) * 64 + lane;
-            const bool live = p < npos;
-            int t = -1, poff = 0;
-            float val = 0.f;
-            long o = 0;
-            if (live) {
-                o = y_off(s, b, g, n, hw0 + p);
-                t = pos[o];
-                const float v = out[o];
-                val = lower ? -v : v;
-                const int pr = small_div(p, OW, rg.inv_ow), pc = p - pr * OW;
-                poff = pr * pm.sh * rg.pitch + pc * pm.sw;
-                if (t < 0 || t >= rg.nt) t = -1;
+    for (int it = wave; it < total; it += nwave) {
+        const int n = it / nmacro, p = (it - n * nmacro) * 64 + lane;
+        const bool live = p < npos;
+        int t1st = -1, t2nd = -1, poff = 0;
+        float val1 = 0.f, val2 = 0.f;
+        long o = 0;
+        if (live) {
+            o = y_off(s, b, g, n, hw0 + p);
+            t1st = pos1[o];
+            val1 = BOUND ? -out1[o] : out1[o];
+            if (t1st < 0 || t1st >= rg.nt) t1st = -1;
+            if constexpr (BOUND) {
+                t2nd = pos2[o];
+                val2 = out2[o];
+                if (t2nd < 0 || t2nd >= rg.nt) t2nd = -1;
             }
-            const float* __restrict__ wrow = w + w_off(s, g, n, 0);
-            uint32_t mine = kNoKey;  // the result of the output this lane read
-            auto step = [&](auto sub_c) __attribute__((always_inline)) {
-                constexpr int sub = decltype(sub_c)::value;
-                constexpr int ctrl = sub | (sub << 2) | (sub << 4) | (sub << 6);  // quad_perm [sub, sub, sub, sub]
-                const int tt = __builtin_amdgcn_update_dpp(0, t, ctrl, 0xf, 0xf, true);
-                const int po = __builtin_amdgcn_update_dpp(0, poff, ctrl, 0xf, 0xf, true);
-                const float target = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(val), ctrl, 0xf, 0xf, true));
-                uint32_t key = kNoKey;
-                if (tt >= 0) {
+            const int pr = small_div(p, OW, rg.inv_ow), pc = p - pr * OW;
+            poff = pr * pm.sh * rg.pitch + pc * pm.sw;
+        }
+        const float* __restrict__ wrow = w + w_off(s, g, n, 0);
+        uint32_t mine1 = kNoKey, mine2 = kNoKey;  // the results of the output this lane read
+        auto step = [&](auto sub_c) __attribute__((always_inline)) {
+            constexpr int sub = decltype(sub_c)::value;
+            constexpr int ctrl = sub | (sub << 2) | (sub << 4) | (sub << 6);  // quad_perm [sub, sub, sub, sub]
+            const int tt1 = __builtin_amdgcn_update_dpp(0, t1st, ctrl, 0xf, 0xf, true);
+            const int po = __builtin_amdgcn_update_dpp(0, poff, ctrl, 0xf, 0xf, true);
+            const float target1 = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(val1), ctrl, 0xf, 0xf, true));
+            int tt2 = -1;
+            float target2 = 0.f;
+            if constexpr (BOUND) {
+                tt2 = __builtin_amdgcn_update_dpp(0, t2nd, ctrl, 0xf, 0xf, true);
+                target2 = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(val2), ctrl, 0xf, 0xf, true));
+            }
+            uint32_t key1 = kNoKey, key2 = kNoKey;
+            // one walk over tile tt: the first output (distance, or lower bound) when `first`, the upper bound when
+            // `second`
+            auto walk = [&](int tt, bool first, bool second) __attribute__((always_inline)) {
 #pragma unroll
-                    for (int h = KT / 16 - 1; h >= 0; h--) {  // descending: the lowest matching k is kept
-                        const int k = tt * KT + (lane & 3) * 4 + 16 * h;
-                        if (k < K) {
-                            float wv[4];
-                            if (w_vec) {
-                                const float4 w4 = *reinterpret_cast<const float4*>(wrow + k);
-                                wv[0] = w4.x; wv[1] = w4.y; wv[2] = w4.z; wv[3] = w4.w;
+                for (int h = KT / 16 - 1; h >= 0; h--) {  // descending: the lowest matching k is kept
+                    const int k = tt * KT + (lane & 3) * 4 + 16 * h;
+                    if (k < K) {
+                        float wv[4];
+                        if (w_vec) {
+                            const float4 w4 = *reinterpret_cast<const float4*>(wrow + k);
+                            wv[0] = w4.x; wv[1] = w4.y; wv[2] = w4.z; wv[3] = w4.w;
+                        } else {
+#pragma unroll
+                            for (int j = 0; j < 4; j++) wv[j] = k + j < K ? wrow[k + j] : 0.f;
+                        }
+                        const int4 tp4 = *reinterpret_cast<const int4*>(tab + k);  // (k is a multiple of four)
+                        const int tp[4] = {tp4.x, tp4.y, tp4.z, tp4.w};
+                        float xa[4], xb[4];  // the reads leave together
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            xa[j] = xs[tp[j] + po];
+                            xb[j] = BOUND ? xs[cg * E + tp[j] + po] : 0.f;
+                        }
+#pragma unroll
+                        for (int j = 3; j >= 0; j--) {
+                            if constexpr (!BOUND) {
+                                const float d = xa[j] - wv[j];
+                                if (fabsf(d) == target1 && k + j < K) key1 = ((uint32_t)(k + j) << 1) | (!(d >= 0) ? 1u : 0u);
                             } else {
-#pragma unroll
-                                for (int j = 0; j < 4; j++) wv[j] = k + j < K ? wrow[k + j] : 0.f;
-                            }
-                            const int4 tp4 = *reinterpret_cast<const int4*>(tab + k);  // (k is a multiple of four)
-                            const int tp[4] = {tp4.x, tp4.y, tp4.z, tp4.w};
-                            float xa[4], xb[4];  // the reads leave together
-#pragma unroll
-                            for (int j = 0; j < 4; j++) {
-                                xa[j] = xs[tp[j] + po];
-                                xb[j] = BOUND ? xs[cg * E + tp[j] + po] : 0.f;
-                            }
-#pragma unroll
-                            for (int j = 3; j >= 0; j--) {
-                                bool hit, neg;
-                                if constexpr (!BOUND) {
-                                    const float d = xa[j] - wv[j];
-                                    hit = fabsf(d) == target;
-                                    neg = !(d >= 0);
-                                } else {
-                                    const float t1 = wv[j] - xa[j], t2 = xb[j] - wv[j];
-                                    hit = (lower ? fminf(t1, t2) : fmaxf(t1, t2)) == target;
-                                    neg = !(t1 <= t2);
-                                }
-                                if (hit && k + j < K) key = ((uint32_t)(k + j) << 1) | (neg ? 1u : 0u);
+                                const float t1 = wv[j] - xa[j], t2 = xb[j] - wv[j];
+                                const uint32_t kk = ((uint32_t)(k + j) << 1) | (!(t1 <= t2) ? 1u : 0u);
+                                if (first && fminf(t1, t2) == target1 && k + j < K) key1 = kk;
+                                if (second && fmaxf(t1, t2) == target2 && k + j < K) key2 = kk;
                             }
                         }
                     }
                 }
-                // lowest key of the four lanes that share the output (all lanes of the wave are here)
-                key = min(key, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)key, 0xB1, 0xf, 0xf, true));   // quad_perm [1,0,3,2]
-                key = min(key, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)key, 0x4E, 0xf, 0xf, true));   // quad_perm [2,3,0,1]
-                if ((lane & 3) == sub) mine = key;
             };
-            step(std::integral_constant<int, 0>{}); step(std::integral_constant<int, 1>{});
-            step(std::integral_constant<int, 2>{}); step(std::integral_constant<int, 3>{});
-            if (live) {
-                uint32_t code = kDefault;
-                if (t >= 0 && mine != kNoKey) code = (mine >> 1) | ((mine & 1u) ? kSignBit : 0u);
-                pos[o] = (int32_t)code;
+            if (tt1 >= 0) walk(tt1, true, BOUND && tt2 == tt1);
+            if constexpr (BOUND) {
+                if (tt2 >= 0 && tt2 != tt1) walk(tt2, false, true);
+            }
+            // lowest key of the four lanes that share the output (all lanes of the wave are here)
+            key1 = min(key1, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)key1, 0xB1, 0xf, 0xf, true));   // quad_perm [1,0,3,2]
+            key1 = min(key1, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)key1, 0x4E, 0xf, 0xf, true));   // quad_perm [2,3,0,1]
+            if ((lane & 3) == sub) mine1 = key1;
+            if constexpr (BOUND) {
+                key2 = min(key2, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)key2, 0xB1, 0xf, 0xf, true));
+                key2 = min(key2, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)key2, 0x4E, 0xf, 0xf, true));
+                if ((lane & 3) == sub) mine2 = key2;
+            }
+        };
+        step(std::integral_constant<int, 0>{}); step(std::integral_constant<int, 1>{});
+        step(std::integral_constant<int, 2>{}); step(std::integral_constant<int, 3>{});
+        if (live) {
+            uint32_t code = BOUND ? kNoGradId : 0u;  // a lower bound of zero has no arg-max
+            if (t1st >= 0 && mine1 != kNoKey) code = (mine1 >> 1) | ((mine1 & 1u) ? kSignBit : 0u);
+            pos1[o] = (int32_t)code;
+            if constexpr (BOUND) {
+                code = 0u;
+                if (t2nd >= 0 && mine2 != kNoKey) code = (mine2 >> 1) | ((mine2 & 1u) ? kSignBit : 0u);
+                pos2[o] = (int32_t)code;
             }
         }
     }
