@@ -236,6 +236,14 @@ def other_workloads(torch, _C, xd, wd, gd):
         y.backward(torch.ones_like(y))
 
     res["conv3x3_128to128_b128_32x32_pinf_fwd_bwd"] = tm(conv_step)
+
+    def conv_ibp_step():  # the layer with its interval bounds at eps = 8/255, forward and backward of all three outputs
+        cx.grad = None
+        conv.weight.grad = None
+        y, lo, up = conv(cx, cx - 8 / 255, cx + 8 / 255)
+        torch.autograd.backward([y, lo, up], [torch.ones_like(y)] * 3)
+
+    res["conv3x3_128to128_b128_32x32_pinf_fwd_bwd_with_ibp"] = tm(conv_ibp_step)
     conv.eval()
     cd = cx.detach()
 
