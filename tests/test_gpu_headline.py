@@ -347,6 +347,65 @@ def test_conv_shape_fused_entry_points():
     assert_close(gw.cpu().numpy(), ew, what="fused conv grad_weight (bounds)")
 
 
+def test_conv_shape_finite_p_entry_points(monkeypatch):
+    # The conv benchmark at p = 8 through the image entry points (reference: F.unfold + norm_dist::forward /
+    # backward_input_weight, core/modules/norm_dist.py:93-102).  Oracle on the patches of three samples: values and
+    # grad_input of those samples through the adjoint of unfold; grad_weight of those three samples alone from a
+    # second call.  Over all 128 samples: the degree-1 homogeneity of the distance,
+    # <grad_x, x> + <grad_w, w> = <grad_out, out> (patches are linear in the image), the sum of grad_weight over the
+    # two halves of the batch, and the two routes of the backward (patches gathered inside the kernel; patches written
+    # out as rows first) giving the same grad_input bit for bit when they walk the batch in the same parts.
+    from core import _C
+    import torch.nn.functional as F
+    gen = torch.Generator().manual_seed(2022)
+    img = torch.randn(128, 128, 32, 32, generator=gen)
+    w = torch.randn(128, 1152, generator=gen) / np.sqrt(1152)
+    g = torch.randn(128, 128, 1024, generator=gen)
+    SAMPLES = [0, 63, 127]
+    P = 8.0
+    geo = (1, P, 3, 1, 1, 1)  # groups, p, kernel, dilation, padding, stride
+    imd, wd, gd = img.cuda(), w.cuda(), g.cuda()
+    patches = F.unfold(img[SAMPLES], 3, 1, 1, 1).numpy()
+    out = torch.empty(128, 128, 1024, device="cuda")
+    _C.conv_norm_dist_forward(imd, wd, out, *geo)
+    assert_close(out[SAMPLES].cpu().numpy(), O.norm_dist_forward(patches, w.numpy(), P), what="conv p=8 forward")
+    gx = torch.full_like(imd, float("nan"))
+    gw = torch.full_like(wd, float("nan"))
+    _C.conv_norm_dist_backward_input_weight(gd, imd, wd, out, gx, gw, *geo)
+    ex_p, ew3 = O.norm_dist_backward(g.numpy()[SAMPLES], patches, w.numpy(), out[SAMPLES].cpu().numpy(), P)
+    ex = F.fold(torch.from_numpy(ex_p), (32, 32), 3, 1, 1, 1).numpy()
+    assert_close(gx[SAMPLES].cpu().numpy(), ex, what="conv p=8 grad_input")
+    sel = torch.tensor(SAMPLES, device="cuda")
+    gx3 = torch.full((3, 128, 32, 32), float("nan"), device="cuda")
+    gw3 = torch.full_like(wd, float("nan"))
+    _C.conv_norm_dist_backward_input_weight(gd[sel].contiguous(), imd[sel].contiguous(), wd, out[sel].contiguous(),
+                                            gx3, gw3, *geo)
+    assert_close(gw3.cpu().numpy(), ew3, what="conv p=8 grad_weight of three samples")
+    assert_close(gx3.cpu().numpy(), ex, what="conv p=8 grad_input of three samples")
+    lhs = (gx.double() * imd.double()).sum().item() + (gw.double() * wd.double()).sum().item()
+    rhs = (gd.double() * out.double()).sum().item()
+    scale = (gd.double().abs() * out.double()).sum().item()
+    assert abs(lhs - rhs) <= 1e-6 * scale, (lhs, rhs, scale)
+    halves = torch.zeros_like(wd, dtype=torch.float64)
+    for h in (slice(0, 64), slice(64, 128)):
+        gxh, gwh = torch.full_like(imd[h], float("nan")), torch.full_like(wd, float("nan"))
+        _C.conv_norm_dist_backward_input_weight(gd[h], imd[h], wd, out[h], gxh, gwh, *geo)
+        assert torch.equal(gxh, gx[h])
+        halves += gwh.double()
+    assert_close(gw.cpu().numpy(), halves.cpu().numpy(), what="conv p=8 grad_weight over the halves of the batch")
+    # (the order of the sums over the output channels depends on how many rows a launch covers: same parts, same bits)
+    monkeypatch.setenv("NORM_DIST_CONV_PART_MB", "128")  # doubled where the kernel gathers: three parts of 43 samples
+    gx_three = torch.full_like(imd, float("nan"))
+    _C.conv_norm_dist_backward_input_weight(gd, imd, wd, out, gx_three, torch.empty_like(wd), *geo)
+    assert_close(gx_three.cpu().numpy(), gx.cpu().numpy(), what="conv p=8 grad_input, three parts")
+    monkeypatch.setenv("NORM_DIST_CONV_PART_MB", "256")  # the default: three parts for the route with two buffers
+    monkeypatch.setenv("NORM_DIST_BWD_GATHER", "0")
+    gx_rows, gw_rows = torch.full_like(imd, float("nan")), torch.full_like(wd, float("nan"))
+    _C.conv_norm_dist_backward_input_weight(gd, imd, wd, out, gx_rows, gw_rows, *geo)
+    assert torch.equal(gx_rows, gx_three)
+    assert_close(gw_rows.cpu().numpy(), gw.cpu().numpy(), what="conv p=8 grad_weight, patches as rows")
+
+
 def test_config4_mlp_step_full_size():
     # MLPModel(depth 6, width 5120) on [512, 3072] uniform inputs, p = 8, hinge loss on the worst-case margins of random
     # labels (reference: ell_inf_models.py:16-46, main.py:304-310): one full forward + backward step.  Every layer's
