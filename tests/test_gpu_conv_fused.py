@@ -347,6 +347,52 @@ def test_conv_codes_with_the_sorted_second_pass(B, C, H, W, CO, G, k, d, p, s, m
     np.testing.assert_array_equal(posu.cpu().numpy(), epu)
 
 
+@pytest.mark.parametrize("B,C,H,W,CO,G,k,d,p,s", [CASES[2], CASES[6], CASES[7]])
+def test_conv_grad_weight_sums_in_fixed_point(B, C, H, W, CO, G, k, d, p, s, monkeypatch):
+    """grad_weight of the scatter backward on images is summed in LDS as 64-bit fixed-point numbers scaled by the
+    largest gradient a workgroup sees; NORM_DIST_SCATTER_FIXED=0 keeps float adds.  Both within 1e-5 of the oracle, for
+    the distance and for the interval bounds; gradients spread over 60 binary orders of magnitude lose nothing that
+    float sums keep; a workgroup that meets an infinity or a NaN falls back to float adds, so they reach the same
+    weights on both routes."""
+    from core import _C
+    x, w = _case(B * 61 + C, B, C, H, W, CO, G, k, d, p, s)
+    patches = F.unfold(x, k, d, p, s)
+    _, ep = O.inf_dist_forward(patches.numpy(), w.numpy(), G)
+    lo, up = x - 0.1, x + 0.1
+    _, _, epl, epu = O.bound_inf_dist_forward(F.unfold(lo, k, d, p, s).numpy(), F.unfold(up, k, d, p, s).numpy(), w.numpy(), G)
+    pos, posl, posu = (torch.from_numpy(a.astype(np.int32)).cuda() for a in (ep, epl, epu))
+    gen = torch.Generator().manual_seed(11)
+    g = torch.randn(ep.shape, generator=gen)
+    g2 = torch.randn(ep.shape, generator=gen)
+    wide = g * torch.exp2(torch.randint(-40, 20, g.shape, generator=gen).float())
+    bad = g.clone()
+    bad[0, 0, 0] = float("inf")
+    bad[-1, -1, -1] = float("nan")
+    results = {}
+    for mode in ("1", "0"):
+        monkeypatch.setenv("NORM_DIST_SCATTER_FIXED", mode)
+        for name, grad in (("plain", g), ("wide", wide), ("bad", bad)):
+            gx, gw = torch.full_like(x.cuda(), float("nan")), torch.full_like(w.cuda(), float("nan"))
+            _C.conv_inf_dist_backward_input_weight(grad.cuda(), pos, gx, gw, G, k, d, p, s)
+            results[mode, name] = gw.cpu().numpy()
+        gxl, gxu = torch.full_like(x.cuda(), float("nan")), torch.full_like(x.cuda(), float("nan"))
+        gwb = torch.full_like(w.cuda(), float("nan"))
+        _C.conv_bound_inf_dist_backward_input_weight(g.cuda(), g2.cuda(), posl, posu, gxl, gxu, gwb, G, k, d, p, s)
+        results[mode, "bounds"] = gwb.cpu().numpy()
+    for name, grad in (("plain", g), ("wide", wide)):
+        _, ew = O.inf_dist_backward(grad.numpy(), ep, patches.size(1), G)
+        for mode in ("1", "0"):
+            assert_close(results[mode, name], ew, what="grad_weight %s, fixed %s" % (name, mode))
+    _, _, ewb = O.bound_inf_dist_backward(g.numpy(), g2.numpy(), epl, epu, patches.size(1), G)
+    for mode in ("1", "0"):
+        assert_close(results[mode, "bounds"], ewb, what="grad_weight of the bounds, fixed %s" % mode)
+    a, b = results["1", "bad"], results["0", "bad"]
+    assert np.array_equal(np.isnan(a), np.isnan(b)) and np.array_equal(np.isinf(a), np.isinf(b))
+    assert np.isnan(a).any() and np.isinf(a).any()
+    fin = np.isfinite(a)
+    assert_close(a[fin], b[fin], what="finite weights beside the non-finite ones")
+
+
 @pytest.mark.parametrize("B,C,H,W,CO,G,k,d,p,s", [CASES[2], CASES[6], CASES[7], TRAIN_CASES[-1], TRAIN_CASES[len(CASES)]])
 def test_conv_backward_by_channel_slabs(B, C, H, W, CO, G, k, d, p, s, monkeypatch):
     """The image gradient of the scatter backward comes from one of two kernels (blocks of output rows where the image
