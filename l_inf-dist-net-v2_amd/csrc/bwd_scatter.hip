@@ -331,85 +331,33 @@ __global__ __launch_bounds__(256) void scatter_gw_split_kernel(const float* __re
     }
 }
 
-// ---- sums in fixed point -----------------------------------------------------------------------------------
-// An LDS float add (ds_add_f32) takes about 190 cycles per wave instruction on this part, a 64-bit integer add 11.
-// Where a workgroup's sums live in LDS and the adds do not pile up on few words, it therefore adds integers: a first
-// pass over its gradients finds their largest magnitude, every value is then scaled by a power of two that leaves
-// `nbits` bits of head room for the number of addends (exact for every value within 2^-(38 - nbits) of the largest,
-// truncated below that), and the sums are converted back once.  The result is the correctly rounded sum to far below
-// float precision, and it does not depend on the order of the adds.  A workgroup that meets an infinity or a NaN
-// falls back to float adds, which propagate them.
-__device__ __forceinline__ long long to_fixed(float v, int shift) {  // trunc(v * 2^shift); zero for subnormal v
-    const unsigned bits = __float_as_uint(v);
-    const int e = (int)((bits >> 23) & 0xffu);
-    if (e == 0) return 0;
-    const long long m = (long long)((bits & 0x7fffffu) | 0x800000u);
-    const int sh = e - 150 + shift;
-    const long long q = sh >= 0 ? (m << sh) : (sh > -24 ? (m >> -sh) : 0ll);
-    return (bits >> 31) ? -q : q;
-}
-__device__ __forceinline__ float from_fixed(long long q, int shift) { return ldexpf((float)q, -shift); }
-__device__ __forceinline__ void lds_add_fixed(long long* acc, int off, float v, int shift) {
-    atomicAdd(reinterpret_cast<unsigned long long*>(acc) + off, (unsigned long long)to_fixed(v, shift));
-}
-// Largest |value| bit pattern over the workgroup (every thread passes its own; `slot` in LDS, zeroed before).
-__device__ __forceinline__ unsigned workgroup_max_bits(unsigned mine, unsigned* slot) {
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) mine = max(mine, (unsigned)__shfl_xor((int)mine, d, 64));
-    if ((threadIdx.x & 63) == 0) atomicMax(slot, mine);
-    __syncthreads();
-    return *slot;
-}
-// shift for values up to the float with magnitude bits `maxbits` (finite), nbits of head room
-__device__ __forceinline__ int fixed_shift(unsigned maxbits, int nbits) { return 62 - nbits - ((int)(maxbits >> 23) - 126); }
-inline int fixed_head_room(long addends) {
-    int n = 1;
-    while ((1L << n) < addends && n < 40) n++;
-    return n + 1;
-}
+// ---- sums in double precision ---------------------------------------------------------------------------------
+// An LDS float add (ds_add_f32) takes about 190 cycles per wave instruction on this part, a double one (ds_add_f64)
+// 21, a 64-bit integer one 11 (measured on random words).  Where a workgroup's sums live in LDS and the adds do not
+// pile up on few words, it therefore adds doubles and rounds once at the end: nine times the rate, and sums that are
+// exact to far below float precision whatever the order of the adds (infinities and NaNs travel as they do in
+// floats).  The price is eight bytes of LDS per sum.
 
-// grad_weight as scatter_gw_split_kernel, sums in fixed point.  LDS: [R][CIg] 64-bit sums.  1024 threads: as many waves
-// per compute unit from a quarter of the workgroups, i.e. a quarter of the adds to global memory at the end.
-constexpr int kGwFixedThreads = 1024;
+// grad_weight as scatter_gw_split_kernel, sums in doubles.  LDS: [R][CIg] doubles.  1024 threads: as many waves per
+// compute unit from a quarter of the workgroups, i.e. a quarter of the adds to global memory at the end.
+constexpr int kGwWideThreads = 1024;
 template <bool BOUND>
-__global__ __launch_bounds__(kGwFixedThreads) void scatter_gw_split_fixed_kernel(const float* __restrict__ g1, const float* __restrict__ g2,
-                                                                     const int32_t* __restrict__ p1,
-                                                                     const int32_t* __restrict__ p2, float* __restrict__ gw,
-                                                                     const Geom s, int R, int nsplit, int nbits) {
-    extern __shared__ long long acc[];  // [R][CIg]
-    __shared__ unsigned wmax;
+__global__ __launch_bounds__(kGwWideThreads) void scatter_gw_split_f64_kernel(const float* __restrict__ g1, const float* __restrict__ g2,
+                                                                              const int32_t* __restrict__ p1,
+                                                                              const int32_t* __restrict__ p2, float* __restrict__ gw,
+                                                                              const Geom s, int R, int nsplit) {
+    extern __shared__ double acc[];  // [R][CIg]
     const int g = blockIdx.y, co0 = blockIdx.x * R, j = blockIdx.z;
     const int nr = min(R, s.COg - co0);
     const int b0 = (int)((long)j * s.B / nsplit), b1 = (int)((long)(j + 1) * s.B / nsplit);
-    if (threadIdx.x == 0) wmax = 0u;
-    for (int i = threadIdx.x; i < nr * s.CIg; i += kGwFixedThreads) acc[i] = 0ll;
+    for (int i = threadIdx.x; i < nr * s.CIg; i += kGwWideThreads) acc[i] = 0.0;
     __syncthreads();
     // A wave takes whole runs -- the HW outputs of one (b, co), contiguous in memory -- with its lanes along hw, and
     // requests the loads of U steps of 64 outputs together: the waves would otherwise wait one memory latency per
     // step, and no index needs a division per output.
     constexpr int U = 8;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwave = kGwFixedThreads / 64;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwave = kGwWideThreads / 64;
     const int nrun = (b1 - b0) * nr;
-    unsigned mx = 0u;
-    for (int t = wave; t < nrun; t += nwave) {
-        const int r = t % nr;
-        const long o0 = y_off(s, b0 + t / nr, g, co0 + r, 0);
-        for (int h0 = 0; h0 < s.HW; h0 += 64 * U) {
-            float ga[U], gb[U];
-#pragma unroll
-            for (int u = 0; u < U; u++) {
-                const int hw = min(h0 + 64 * u + lane, s.HW - 1);
-                ga[u] = g1[o0 + hw];
-                gb[u] = BOUND ? g2[o0 + hw] : 0.f;
-            }
-#pragma unroll
-            for (int u = 0; u < U; u++) mx = max(mx, max(__float_as_uint(ga[u]), __float_as_uint(gb[u])) & 0x7fffffffu);
-        }
-    }
-    mx = workgroup_max_bits(mx, &wmax);
-    const bool finite = (mx >> 23) != 0xffu;
-    const int shift = fixed_shift(mx, nbits);
-    float* __restrict__ rows = reinterpret_cast<float*>(acc);  // the fall-back's sums: zero as well
     for (int t = wave; t < nrun; t += nwave) {
         const int r = t % nr;
         const long o0 = y_off(s, b0 + t / nr, g, co0 + r, 0);
@@ -430,24 +378,18 @@ __global__ __launch_bounds__(kGwFixedThreads) void scatter_gw_split_fixed_kernel
             for (int u = 0; u < U; u++) {
                 if (h0 + 64 * u + lane >= s.HW) continue;
                 const Route a = BOUND ? route_lower(pa[u], ga[u]) : route_inf(pa[u], ga[u]);
-                if (a.target >= 0 && a.idx < s.CIg) {
-                    if (finite) lds_add_fixed(acc, r * s.CIg + a.idx, -a.v, shift);
-                    else atomicAdd(rows + r * s.CIg + a.idx, -a.v);
-                }
+                if (a.target >= 0 && a.idx < s.CIg) atomicAdd(acc + r * s.CIg + a.idx, -(double)a.v);
                 if (BOUND) {
                     const Route c = route_upper(pb[u], gb[u]);
-                    if (c.idx < s.CIg) {
-                        if (finite) lds_add_fixed(acc, r * s.CIg + c.idx, -c.v, shift);
-                        else atomicAdd(rows + r * s.CIg + c.idx, -c.v);
-                    }
+                    if (c.idx < s.CIg) atomicAdd(acc + r * s.CIg + c.idx, -(double)c.v);
                 }
             }
         }
     }
     __syncthreads();
     float* dst = gw + w_off(s, g, co0, 0);
-    for (int i = threadIdx.x; i < nr * s.CIg; i += kGwFixedThreads) {
-        const float v = finite ? from_fixed(acc[i], shift) : rows[i];
+    for (int i = threadIdx.x; i < nr * s.CIg; i += kGwWideThreads) {
+        const float v = (float)acc[i];
         if (nsplit == 1) dst[i] = v;
         else if (v != 0.f) atomicAdd(dst + i, v);
     }
@@ -733,9 +675,9 @@ __global__ __launch_bounds__(1024) void scatter_gx_ownrows_kernel(const float* _
     }
 }
 
-// NORM_DIST_SCATTER_FIXED=0: float adds in LDS everywhere (tuning / test aid, read at every call)
-static bool scatter_fixed_enabled() {
-    const char* e = getenv("NORM_DIST_SCATTER_FIXED");
+// NORM_DIST_SCATTER_F64=0: float adds in LDS everywhere (tuning / test aid, read at every call)
+static bool scatter_f64_enabled() {
+    const char* e = getenv("NORM_DIST_SCATTER_F64");
     return e == nullptr || e[0] != '0';
 }
 constexpr int kScatterLdsBudget = 96 * 1024;
@@ -752,25 +694,23 @@ static int scatter_backward_images(const float* g1, const float* g2, const int32
     if (gw && (size_t)s.CIg * sizeof(float) > (size_t)kScatterLdsBudget) return -1;
     // grad_weight launch parameters (shared by both grad_input routes)
     int R = 1, ncb = 0, nsplit = 1;
-    const bool gw_fixed = scatter_fixed_enabled() && (size_t)s.CIg * sizeof(long long) <= (size_t)kScatterLdsBudget;
+    const bool gw_wide = scatter_f64_enabled() && (size_t)s.CIg * sizeof(double) <= (size_t)kScatterLdsBudget;
     auto prepare_gw = [&]() -> int {
-        NDIST_HIP_TRY(hipFuncSetAttribute(gw_fixed ? reinterpret_cast<const void*>(&scatter_gw_split_fixed_kernel<BOUND>)
+        NDIST_HIP_TRY(hipFuncSetAttribute(gw_wide ? reinterpret_cast<const void*>(&scatter_gw_split_f64_kernel<BOUND>)
                                                    : reinterpret_cast<const void*>(&scatter_gw_split_kernel<BOUND>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, kScatterLdsBudget));
-        R = (int)((size_t)kScatterLdsBudget / ((size_t)s.CIg * (gw_fixed ? sizeof(long long) : sizeof(float))));
+        R = (int)((size_t)kScatterLdsBudget / ((size_t)s.CIg * (gw_wide ? sizeof(double) : sizeof(float))));
         R = R > 4 ? 4 : R;
         ncb = ceil_div(s.COg, R);
-        nsplit = ceil_div((gw_fixed ? 1 : 4) * device_info().num_cu, ncb * s.G);
+        nsplit = ceil_div((gw_wide ? 1 : 4) * device_info().num_cu, ncb * s.G);
         nsplit = nsplit > s.B ? s.B : nsplit;
         nsplit = nsplit > 65535 ? 65535 : nsplit;
         return nsplit > 1 ? fill_zero(gw, (long)s.COg * s.G * s.CIg, st) : 0;
     };
     auto launch_gw = [&]() -> int {
-        if (gw_fixed) {
-            // addends per sum: every output of a workgroup's share of the batch could name the same weight
-            const int nbits = fixed_head_room((long)ceil_div(s.B, nsplit) * s.HW * (BOUND ? 2 : 1));
-            hipLaunchKernelGGL(scatter_gw_split_fixed_kernel<BOUND>, dim3(ncb, s.G, nsplit), dim3(kGwFixedThreads),
-                               (size_t)R * s.CIg * sizeof(long long), st, g1, g2, p1, p2, gw, s, R, nsplit, nbits);
+        if (gw_wide) {
+            hipLaunchKernelGGL(scatter_gw_split_f64_kernel<BOUND>, dim3(ncb, s.G, nsplit), dim3(kGwWideThreads),
+                               (size_t)R * s.CIg * sizeof(double), st, g1, g2, p1, p2, gw, s, R, nsplit);
         } else {
             hipLaunchKernelGGL(scatter_gw_split_kernel<BOUND>, dim3(ncb, s.G, nsplit), dim3(256),
                                (size_t)R * s.CIg * sizeof(float), st, g1, g2, p1, p2, gw, s, R, nsplit);
@@ -889,17 +829,17 @@ static int scatter_backward(const float* g1, const float* g2, const int32_t* p1,
         if (nslab <= 8 && nwg < (1L << 31)) {
             NDIST_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&scatter_gx_tile_kernel<BOUND>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, kScatterTileBudget));
-            // (sums in fixed point where a row of 64-bit sums fits: see scatter_gw_split_fixed_kernel)
-            const bool gw_fixed = scatter_fixed_enabled() && (size_t)s.CIg * sizeof(long long) <= (size_t)kScatterLdsBudget;
-            NDIST_HIP_TRY(hipFuncSetAttribute(gw_fixed ? reinterpret_cast<const void*>(&scatter_gw_split_fixed_kernel<BOUND>)
+            // (sums in doubles where a row of them fits: see scatter_gw_split_f64_kernel)
+            const bool gw_wide = scatter_f64_enabled() && (size_t)s.CIg * sizeof(double) <= (size_t)kScatterLdsBudget;
+            NDIST_HIP_TRY(hipFuncSetAttribute(gw_wide ? reinterpret_cast<const void*>(&scatter_gw_split_f64_kernel<BOUND>)
                                                        : reinterpret_cast<const void*>(&scatter_gw_split_kernel<BOUND>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, kScatterLdsBudget));
-            int R = (int)((size_t)kScatterLdsBudget / ((size_t)s.CIg * (gw_fixed ? sizeof(long long) : sizeof(float))));
+            int R = (int)((size_t)kScatterLdsBudget / ((size_t)s.CIg * (gw_wide ? sizeof(double) : sizeof(float))));
             R = R > 4 ? 4 : R;
             const int ncb = ceil_div(s.COg, R);
             // enough workgroups to cover the device about four times (once with the 1024-thread workgroups of the
-            // fixed-point kernel), at most one share per sample
-            int nsplit = ceil_div((gw_fixed ? 1 : 4) * device_info().num_cu, ncb * s.G);
+            // kernel that sums in doubles), at most one share per sample
+            int nsplit = ceil_div((gw_wide ? 1 : 4) * device_info().num_cu, ncb * s.G);
             nsplit = nsplit > s.B ? s.B : nsplit;
             nsplit = nsplit > 65535 ? 65535 : nsplit;
             if (gw && nsplit > 1) {
@@ -911,10 +851,9 @@ static int scatter_backward(const float* g1, const float* g2, const int32_t* p1,
                                (size_t)nx * CS * kScatterHB * sizeof(float), st, g1, g2, p1, p2, gx1, gx2, s, CS, nslab,
                                nhb);
             if (hip_failed(hipGetLastError())) return 4;
-            if (gw && gw_fixed) {
-                const int nbits = fixed_head_room((long)ceil_div(s.B, nsplit) * s.HW * (BOUND ? 2 : 1));
-                hipLaunchKernelGGL(scatter_gw_split_fixed_kernel<BOUND>, dim3(ncb, s.G, nsplit), dim3(kGwFixedThreads),
-                                   (size_t)R * s.CIg * sizeof(long long), st, g1, g2, p1, p2, gw, s, R, nsplit, nbits);
+            if (gw && gw_wide) {
+                hipLaunchKernelGGL(scatter_gw_split_f64_kernel<BOUND>, dim3(ncb, s.G, nsplit), dim3(kGwWideThreads),
+                                   (size_t)R * s.CIg * sizeof(double), st, g1, g2, p1, p2, gw, s, R, nsplit);
                 if (hip_failed(hipGetLastError())) return 4;
             } else if (gw) {
                 hipLaunchKernelGGL(scatter_gw_split_kernel<BOUND>, dim3(ncb, s.G, nsplit), dim3(256),

@@ -348,12 +348,11 @@ def test_conv_codes_with_the_sorted_second_pass(B, C, H, W, CO, G, k, d, p, s, m
 
 
 @pytest.mark.parametrize("B,C,H,W,CO,G,k,d,p,s", [CASES[2], CASES[6], CASES[7]])
-def test_conv_grad_weight_sums_in_fixed_point(B, C, H, W, CO, G, k, d, p, s, monkeypatch):
-    """grad_weight of the scatter backward on images is summed in LDS as 64-bit fixed-point numbers scaled by the
-    largest gradient a workgroup sees; NORM_DIST_SCATTER_FIXED=0 keeps float adds.  Both within 1e-5 of the oracle, for
-    the distance and for the interval bounds; gradients spread over 60 binary orders of magnitude lose nothing that
-    float sums keep; a workgroup that meets an infinity or a NaN falls back to float adds, so they reach the same
-    weights on both routes."""
+def test_conv_grad_weight_sums_in_doubles(B, C, H, W, CO, G, k, d, p, s, monkeypatch):
+    """grad_weight of the scatter backward on images is summed in LDS in double precision (nine times the rate of
+    float adds on this part) and rounded once; NORM_DIST_SCATTER_F64=0 keeps float adds.  Both within 1e-5 of the
+    oracle, for the distance and for the interval bounds, also on gradients spread over 60 binary orders of
+    magnitude; infinities and NaNs reach the same weights on both routes."""
     from core import _C
     x, w = _case(B * 61 + C, B, C, H, W, CO, G, k, d, p, s)
     patches = F.unfold(x, k, d, p, s)
@@ -370,7 +369,7 @@ def test_conv_grad_weight_sums_in_fixed_point(B, C, H, W, CO, G, k, d, p, s, mon
     bad[-1, -1, -1] = float("nan")
     results = {}
     for mode in ("1", "0"):
-        monkeypatch.setenv("NORM_DIST_SCATTER_FIXED", mode)
+        monkeypatch.setenv("NORM_DIST_SCATTER_F64", mode)
         for name, grad in (("plain", g), ("wide", wide), ("bad", bad)):
             gx, gw = torch.full_like(x.cuda(), float("nan")), torch.full_like(w.cuda(), float("nan"))
             _C.conv_inf_dist_backward_input_weight(grad.cuda(), pos, gx, gw, G, k, d, p, s)
@@ -382,10 +381,10 @@ def test_conv_grad_weight_sums_in_fixed_point(B, C, H, W, CO, G, k, d, p, s, mon
     for name, grad in (("plain", g), ("wide", wide)):
         _, ew = O.inf_dist_backward(grad.numpy(), ep, patches.size(1), G)
         for mode in ("1", "0"):
-            assert_close(results[mode, name], ew, what="grad_weight %s, fixed %s" % (name, mode))
+            assert_close(results[mode, name], ew, what="grad_weight %s, doubles %s" % (name, mode))
     _, _, ewb = O.bound_inf_dist_backward(g.numpy(), g2.numpy(), epl, epu, patches.size(1), G)
     for mode in ("1", "0"):
-        assert_close(results[mode, "bounds"], ewb, what="grad_weight of the bounds, fixed %s" % mode)
+        assert_close(results[mode, "bounds"], ewb, what="grad_weight of the bounds, doubles %s" % mode)
     a, b = results["1", "bad"], results["0", "bad"]
     assert np.array_equal(np.isnan(a), np.isnan(b)) and np.array_equal(np.isinf(a), np.isinf(b))
     assert np.isnan(a).any() and np.isinf(a).any()
