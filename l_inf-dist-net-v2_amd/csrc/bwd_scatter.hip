@@ -583,13 +583,14 @@ struct ImageRowOwners {
     int nib;   // row blocks per sample
     float inv_ow;
 };
-template <bool BOUND>
+// ACC: float, or double where the rows still fit then (see "sums in double precision" above).
+template <bool BOUND, typename ACC>
 __global__ __launch_bounds__(1024) void scatter_gx_ownrows_kernel(const float* __restrict__ g1, const float* __restrict__ g2,
                                                                  const int32_t* __restrict__ p1,
                                                                  const int32_t* __restrict__ p2, float* __restrict__ gx1,
                                                                  float* __restrict__ gx2, const Geom s, const PatchMap pm,
                                                                  const ImageRowOwners ro) {
-    extern __shared__ float lds[];
+    extern __shared__ __align__(16) float lds[];
     constexpr int NX = BOUND ? 2 : 1;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), nwave = (int)blockDim.x >> 6, nthr = (int)blockDim.x;
@@ -600,7 +601,7 @@ __global__ __launch_bounds__(1024) void scatter_gx_ownrows_kernel(const float* _
     const int cg = pm.cg, K = s.CIg, OW = pm.OW, OH = s.HW / pm.OW, W = pm.W, RI = ro.RI;
     const int K4 = (K + 3) & ~3, kh = pm.taps / pm.kw;
     int* __restrict__ tab = reinterpret_cast<int*>(lds);  // [K4]
-    float* __restrict__ acc = lds + K4;                    // [NX][cg][RI][W]
+    ACC* __restrict__ acc = reinterpret_cast<ACC*>(lds + K4);  // [NX][cg][RI][W]  (K4 floats: 16-byte aligned)
     const int r0 = ib * RI, rows = min(RI, pm.H - r0), cell = RI * W;
     // output rows whose windows reach the rows [r0, r0 + rows)
     const int lo_num = r0 + pm.ph - (kh - 1) * pm.dh;
@@ -608,7 +609,7 @@ __global__ __launch_bounds__(1024) void scatter_gx_ownrows_kernel(const float* _
     const int oh_hi = min(OH - 1, (r0 + rows - 1 + pm.ph) / pm.sh);
     const int npos = oh_hi >= oh_lo ? (oh_hi - oh_lo + 1) * OW : 0, hw0 = oh_lo * OW;
     for (int k = tid; k < K; k += nthr) tab[k] = pack_tap(patch_tap(pm, 0, k));
-    for (int i = tid; i < NX * cg * cell; i += nthr) acc[i] = 0.f;
+    for (int i = tid; i < NX * cg * cell; i += nthr) acc[i] = (ACC)0;
     __syncthreads();
 
     const int nmacro = (npos + 63) >> 6;
@@ -619,7 +620,7 @@ __global__ __launch_bounds__(1024) void scatter_gx_ownrows_kernel(const float* _
         const PatchTap t = unpack_tap(tab[a.idx]);
         const int row = rowbase + t.dy, col = colbase + t.dx;
         if ((unsigned)row < (unsigned)rows && (unsigned)col < (unsigned)W)
-            atomicAdd(&acc[(a.target * cg + t.ch) * cell + row * W + col], a.v);
+            atomicAdd(&acc[(a.target * cg + t.ch) * cell + row * W + col], (ACC)a.v);
     };
 #pragma unroll 1
     for (int it0 = wave; it0 < total; it0 += nwave * UN) {
@@ -657,20 +658,21 @@ __global__ __launch_bounds__(1024) void scatter_gx_ownrows_kernel(const float* _
     const int n = rows * W;
     const bool vec = n % 4 == 0 && cell % 4 == 0 && plane % 4 == 0 && (r0 * W) % 4 == 0 && (uintptr_t)gx1 % 16 == 0 &&
                      (!BOUND || (uintptr_t)gx2 % 16 == 0);
+    auto sum4 = [&](int off) -> float4 {
+        return make_float4((float)acc[off], (float)acc[off + 1], (float)acc[off + 2], (float)acc[off + 3]);
+    };
     if (vec) {
         const int n4 = n / 4;
         for (int i = tid; i < cg * n4; i += nthr) {
             const int c = i / n4, e = (i - c * n4) * 4;
-            *reinterpret_cast<float4*>(gx1 + img + c * plane + e) = *reinterpret_cast<const float4*>(acc + c * cell + e);
-            if (BOUND)
-                *reinterpret_cast<float4*>(gx2 + img + c * plane + e) =
-                    *reinterpret_cast<const float4*>(acc + (cg + c) * cell + e);
+            *reinterpret_cast<float4*>(gx1 + img + c * plane + e) = sum4(c * cell + e);
+            if (BOUND) *reinterpret_cast<float4*>(gx2 + img + c * plane + e) = sum4((cg + c) * cell + e);
         }
     } else {
         for (int i = tid; i < cg * n; i += nthr) {
             const int c = i / n, e = i - c * n;
-            gx1[img + c * plane + e] = acc[c * cell + e];
-            if (BOUND) gx2[img + c * plane + e] = acc[(cg + c) * cell + e];
+            gx1[img + c * plane + e] = (float)acc[c * cell + e];
+            if (BOUND) gx2[img + c * plane + e] = (float)acc[(cg + c) * cell + e];
         }
     }
 }
@@ -725,25 +727,39 @@ static int scatter_backward_images(const float* g1, const float* g2, const int32
     if ((sw == nullptr || (sw[0] != '0' && sw[0] != '1')) && pm.packable && s.CIg <= kRiMaxK && pm.OW > 0) {
         const int kh = pm.taps / pm.kw, reach = (kh - 1) * pm.dh;
         const size_t tabb = (size_t)((s.CIg + 3) & ~3) * sizeof(float);
-        const size_t per_row = (size_t)nx * pm.cg * pm.W * sizeof(float);
         const int want = std::max(2 * reach, 1);
-        int RI = (int)(((size_t)kRiLdsBudget / 2 - tabb) / per_row), threads = 512;
-        if (RI < want) {
-            RI = (int)(((size_t)kRiLdsBudget - tabb) / per_row);
-            threads = 1024;
+        // sums in doubles where a block of rows still fits then, else in floats
+        bool wide = scatter_f64_enabled();
+        size_t per_row = 0;
+        int RI = 0, threads = 512;
+        for (int attempt = 0; attempt < 2; attempt++) {
+            per_row = (size_t)nx * pm.cg * pm.W * (wide ? sizeof(double) : sizeof(float));
+            RI = (int)(((size_t)kRiLdsBudget / 2 - tabb) / per_row);
+            threads = 512;
+            if (RI < want) {
+                RI = (int)(((size_t)kRiLdsBudget - tabb) / per_row);
+                threads = 1024;
+            }
+            RI = std::min(RI, pm.H);
+            if (!wide || RI >= want || RI == pm.H) break;
+            wide = false;
         }
-        RI = std::min(RI, pm.H);
         const long nwg = RI > 0 ? (long)s.B * s.G * ceil_div(pm.H, RI) : 0;
         if ((RI >= want || RI == pm.H) && RI > 0 && nwg < (1L << 31)) {
             const ImageRowOwners ro{RI, ceil_div(pm.H, RI), 1.0f / (float)pm.OW};
-            NDIST_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&scatter_gx_ownrows_kernel<BOUND>),
-                                              hipFuncAttributeMaxDynamicSharedMemorySize, kRiLdsBudget));
+            const void* kern = wide ? reinterpret_cast<const void*>(&scatter_gx_ownrows_kernel<BOUND, double>)
+                                    : reinterpret_cast<const void*>(&scatter_gx_ownrows_kernel<BOUND, float>);
+            NDIST_HIP_TRY(hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, kRiLdsBudget));
             if (gw) {
                 if (int rc = prepare_gw()) return rc;
             }
             KernelTimer timer(st);  // both kernels together
-            hipLaunchKernelGGL(scatter_gx_ownrows_kernel<BOUND>, dim3((unsigned)nwg), dim3(threads),
-                               tabb + (size_t)RI * per_row, st, g1, g2, p1, p2, gx1, gx2, s, pm, ro);
+            if (wide)
+                hipLaunchKernelGGL((scatter_gx_ownrows_kernel<BOUND, double>), dim3((unsigned)nwg), dim3(threads),
+                                   tabb + (size_t)RI * per_row, st, g1, g2, p1, p2, gx1, gx2, s, pm, ro);
+            else
+                hipLaunchKernelGGL((scatter_gx_ownrows_kernel<BOUND, float>), dim3((unsigned)nwg), dim3(threads),
+                                   tabb + (size_t)RI * per_row, st, g1, g2, p1, p2, gx1, gx2, s, pm, ro);
             if (hip_failed(hipGetLastError())) return 4;
             return gw ? launch_gw() : 0;
         }
