@@ -96,7 +96,8 @@ __device__ __forceinline__ float wave_sum(float v) {
     return (__builtin_bit_cast(float, __builtin_amdgcn_readlane(i, 0)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(i, 16))) +
            (__builtin_bit_cast(float, __builtin_amdgcn_readlane(i, 32)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(i, 48)));
 }
-__device__ __forceinline__ void lds_add_clustered(float* base, int off, float v) {
+template <typename ACC>
+__device__ __forceinline__ void lds_add_clustered(ACC* base, int off, float v) {
     const int lane = threadIdx.x & 63;
     bool active = off >= 0;
 #pragma unroll 1
@@ -109,32 +110,30 @@ __device__ __forceinline__ void lds_add_clustered(float* base, int off, float v)
         const unsigned long long grp = __builtin_amdgcn_ballot_w64(mine);
         if (__builtin_popcountll(grp) < 8) break;
         const float sum = wave_sum(mine ? v : 0.f);
-        if (lane == leader) atomicAdd(base + loff, sum);
+        if (lane == leader) atomicAdd(base + loff, (ACC)sum);
         active = active && !mine;
     }
-    if (active) atomicAdd(base + off, v);
+    if (active) atomicAdd(base + off, (ACC)v);
 }
 
 constexpr int kScatterBatch = 8;  // outputs whose codes and gradients a thread requests before it adds any of them
 
 // ---- privatised path, HW == 1 ---------------------------------------------------------------------------
 // grad_input: one workgroup per (b, g); LDS holds the CIg-long row (two rows for the interval variant).
-template <bool BOUND>
+// ACC: float, or double (LDS double adds run at nine times the rate of float ones on this part, see below).
+template <bool BOUND, typename ACC>
 __global__ __launch_bounds__(1024) void scatter_gx_rows_kernel(const float* __restrict__ g1, const float* __restrict__ g2,
                                                               const int32_t* __restrict__ p1,
                                                               const int32_t* __restrict__ p2, float* __restrict__ gx1,
                                                               float* __restrict__ gx2, const Geom s) {
-    extern __shared__ float row[];  // [BOUND ? 2 : 1][CIg]
+    extern __shared__ __align__(16) float row_lds[];
+    ACC* __restrict__ row = reinterpret_cast<ACC*>(row_lds);  // [BOUND ? 2 : 1][CIg]
     const int b = blockIdx.x, g = blockIdx.y, nt = blockDim.x;
     const int nrow = (BOUND ? 2 : 1) * s.CIg;
     const long xbase = x_off(s, b, g, 0, 0);
     // 16-byte LDS and global accesses when the rows allow it (the dynamic LDS base is 16-byte aligned)
     const bool vec = s.CIg % 4 == 0 && (uintptr_t)(gx1 + xbase) % 16 == 0 && (!BOUND || (uintptr_t)(gx2 + xbase) % 16 == 0);
-    if (vec) {
-        for (int i = threadIdx.x; i < nrow / 4; i += nt) reinterpret_cast<float4*>(row)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-    } else {
-        for (int i = threadIdx.x; i < nrow; i += nt) row[i] = 0.f;
-    }
+    for (int i = threadIdx.x; i < nrow; i += nt) row[i] = (ACC)0;
     __syncthreads();
     const long obase = y_off(s, b, g, 0, 0);
     // the loads of kScatterBatch outputs are issued together: one memory latency per batch, not per output
@@ -168,14 +167,15 @@ __global__ __launch_bounds__(1024) void scatter_gx_rows_kernel(const float* __re
     }
     __syncthreads();
     if (vec) {
+        auto sum4 = [&](int e) { return make_float4((float)row[e], (float)row[e + 1], (float)row[e + 2], (float)row[e + 3]); };
         for (int i = threadIdx.x; i < s.CIg / 4; i += nt) {
-            reinterpret_cast<float4*>(gx1 + xbase)[i] = reinterpret_cast<const float4*>(row)[i];
-            if (BOUND) reinterpret_cast<float4*>(gx2 + xbase)[i] = reinterpret_cast<const float4*>(row + s.CIg)[i];
+            reinterpret_cast<float4*>(gx1 + xbase)[i] = sum4(4 * i);
+            if (BOUND) reinterpret_cast<float4*>(gx2 + xbase)[i] = sum4(s.CIg + 4 * i);
         }
     } else {
         for (int i = threadIdx.x; i < s.CIg; i += nt) {
-            gx1[xbase + i] = row[i];
-            if (BOUND) gx2[xbase + i] = row[s.CIg + i];
+            gx1[xbase + i] = (float)row[i];
+            if (BOUND) gx2[xbase + i] = (float)row[s.CIg + i];
         }
     }
 }
@@ -810,15 +810,22 @@ static int scatter_backward(const float* g1, const float* g2, const int32_t* p1,
     const int nx = BOUND ? 2 : 1;
     const size_t gx_lds = (size_t)nx * s.CIg * sizeof(float);
     if (s.HW == 1 && gx_lds <= (size_t)kScatterLdsBudget) {
-        NDIST_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&scatter_gx_rows_kernel<BOUND>),
+        const bool gx_wide = scatter_f64_enabled() && 2 * gx_lds <= (size_t)kScatterLdsBudget;
+        NDIST_HIP_TRY(hipFuncSetAttribute(gx_wide ? reinterpret_cast<const void*>(&scatter_gx_rows_kernel<BOUND, double>)
+                                                  : reinterpret_cast<const void*>(&scatter_gx_rows_kernel<BOUND, float>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, kScatterLdsBudget));
         NDIST_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&scatter_gw_rows_kernel<BOUND>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, kScatterLdsBudget));
         KernelTimer timer(st);  // both row kernels together
         // a row of 2048 outputs and more gets 1024 threads: the kernel has one workgroup per batch row and lives on
         // how many loads each of them keeps in flight
-        hipLaunchKernelGGL(scatter_gx_rows_kernel<BOUND>, dim3(s.B, s.G), dim3(s.COg >= 2048 ? 1024 : 256), gx_lds, st, g1, g2,
-                           p1, p2, gx1, gx2, s);
+        const dim3 gx_grid(s.B, s.G), gx_block(s.COg >= 2048 ? 1024 : 256);
+        if (gx_wide)
+            hipLaunchKernelGGL((scatter_gx_rows_kernel<BOUND, double>), gx_grid, gx_block, 2 * gx_lds, st, g1, g2, p1, p2,
+                               gx1, gx2, s);
+        else
+            hipLaunchKernelGGL((scatter_gx_rows_kernel<BOUND, float>), gx_grid, gx_block, gx_lds, st, g1, g2, p1, p2, gx1,
+                               gx2, s);
         if (hip_failed(hipGetLastError())) return 4;
         if (gw) {
             int R = (int)((size_t)kScatterLdsBudget / ((size_t)s.CIg * sizeof(float)));
