@@ -741,11 +741,11 @@ static int scatter_backward_images(const float* g1, const float* g2, const int32
                 threads = 1024;
             }
             RI = std::min(RI, pm.H);
-            if (!wide || RI >= want || RI == pm.H) break;
+            if (!wide || RI >= (nx == 2 ? std::max(reach, 1) : want) || RI == pm.H) break;
             wide = false;
         }
         const long nwg = RI > 0 ? (long)s.B * s.G * ceil_div(pm.H, RI) : 0;
-        if ((RI >= want || RI == pm.H) && RI > 0 && nwg < (1L << 31)) {
+        if ((RI >= want || RI == pm.H || (wide && nx == 2 && RI >= std::max(reach, 1))) && RI > 0 && nwg < (1L << 31)) {
             const ImageRowOwners ro{RI, ceil_div(pm.H, RI), 1.0f / (float)pm.OW};
             const void* kern = wide ? reinterpret_cast<const void*>(&scatter_gx_ownrows_kernel<BOUND, double>)
                                     : reinterpret_cast<const void*>(&scatter_gx_ownrows_kernel<BOUND, float>);
